@@ -164,6 +164,9 @@ def load_hf_config(model: str, overrides: Optional[dict] = None) -> HFConfig:
     if d.get("model_type") in ("bart", "mbart") and "hidden_size" not in d:
         d = {**d, "hidden_size": d["d_model"], "num_attention_heads": d["decoder_attention_heads"],
              "num_key_value_heads": d["decoder_attention_heads"], "num_hidden_layers": d["decoder_layers"]}
+    if d.get("architecture") == "Nositar":         # a layer-list configuration with names of its own
+        from .models.nositar import normalise_config as nositar_config
+        d = nositar_config(d, model if os.path.isdir(model) else None)
     if d.get("model_type") in ("exaone", "telechat", "qwen", "chatglm"):
         from .models.renamed_decoders import normalise_config
         d = normalise_config(d)
@@ -331,7 +334,7 @@ class ModelConfig:
                          # encoder-decoder: the cross-attention cache is per-request state of the same kind
                          "WhisperForConditionalGeneration", "BartForConditionalGeneration", "BartModel",
                          "MllamaForConditionalGeneration", "Zamba2ForCausalLM", "Plamo2ForCausalLM",
-                         "Florence2ForConditionalGeneration")
+                         "Florence2ForConditionalGeneration", "NositarForCausalLM")
                    for a in self.architectures)
 
     @property

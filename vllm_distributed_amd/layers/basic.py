@@ -73,6 +73,17 @@ class GeluAndMul(nn.Module):
         return ops.act_and_mul(x, self.kind)
 
 
+class ActAndMul(nn.Module):
+    """act(x[..., :d]) * x[..., d:] for any activation the fused kernel knows (ReLU-gated MLPs)."""
+
+    def __init__(self, kind: str):
+        super().__init__()
+        self.kind = kind
+
+    def forward(self, x):
+        return ops.act_and_mul(x, self.kind)
+
+
 class MulAndSilu(nn.Module):
     def forward(self, x):
         return ops.act_and_mul(x, "silu", act_first=False)
@@ -115,6 +126,8 @@ def get_act_and_mul_fn(name: str) -> nn.Module:
         return GeluAndMul()
     if name in ("gelu_tanh", "gelu_pytorch_tanh"):
         return GeluAndMul("tanh")
+    if name in ("relu", "relu2"):
+        return ActAndMul(name)
     raise ValueError(f"unsupported gated activation {name!r}")
 
 

@@ -1252,3 +1252,113 @@ def lightning_attention_decode(qkv: torch.Tensor, state: torch.Tensor, slope: to
     live = (seq_lens[:S] > 0).view(S, 1, 1, 1)
     state[slots] = torch.where(live, s, state[slots])
     return torch.matmul(q.unsqueeze(-2), s).squeeze(-2)
+
+
+# ---- residual streams (hyper-connections) ---------------------------------------------------------------
+def stream_embed(ids: torch.Tensor, weight: torch.Tensor, scale: float, streams: int) -> torch.Tensor:
+    """fp32 residual streams [streams, T, W], each ``weight[ids] * scale``."""
+    if not _dev(weight):
+        return R.stream_embed(ids, weight, scale, streams)
+    T, W = ids.shape[0], weight.shape[1]
+    xs = torch.empty((streams, T, W), dtype=torch.float32, device=weight.device)
+    ids = ids if ids.dtype == torch.int32 else ids.to(torch.int32)
+    N.call("vda_stream_embed", xs.data_ptr(), ids.data_ptr(), weight.data_ptr(), float(scale), T, W, streams,
+           xs.stride(0), N.dt(weight.dtype), N.stream())
+    return xs
+
+
+def stream_step(xs: torch.Tensor, y: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                w_out: Optional[torch.Tensor] = None, w_in: Optional[torch.Tensor] = None,
+                gain: Optional[torch.Tensor] = None, eps: float = 1e-6,
+                out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """One pass over the fp32 residual streams ``xs`` [n, T, W]:
+    write (``y`` given):  xs[t] <- sum_s mix[s, t] xs[s] + w_out[t] y, in place, all streams from the old ones;
+    read (``w_in`` given): returns u / sqrt(mean(u^2) + eps) * gain with u = sum_s w_in[s] xs[s] (after the write),
+    one gain for the whole row.  mix, w_out, w_in, gain are fp32 tensors."""
+    n, T, W = xs.shape
+    if not _dev(xs):
+        if y is not None:
+            R.stream_update(xs, y, mix, w_out)
+        return R.stream_mix_norm(xs, w_in, gain, eps, out_dtype) if w_in is not None else None
+    assert xs.dtype == torch.float32 and xs.is_contiguous()
+    h = None
+    if w_in is not None:
+        h = torch.empty((T, W), dtype=out_dtype, device=xs.device)
+    if y is not None:
+        assert y.stride(1) == 1 and y.shape == (T, W)
+    N.call("vda_stream_step", xs.data_ptr(), N.ptr(y), y.stride(0) if y is not None else 0, N.ptr(mix), N.ptr(w_out),
+           N.ptr(h), N.ptr(w_in), N.ptr(gain), float(eps), T, W, n, xs.stride(0),
+           N.dt(y.dtype) if y is not None else 0, N.dt(h.dtype) if h is not None else 0, N.stream())
+    return h
+
+
+# ---- sigmoid attention with mixed head scores --------------------------------------------------------------
+def unit_rms_qk_and_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, eps: float,
+                          k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                          slot_mapping: torch.Tensor) -> torch.Tensor:
+    """qkv [T, H*D + G*D + G*Dv]: returns q / rms(q) per head (fp32 [T, H, D]) and stores k / rms(k) and v in the
+    paged cache (k_cache [blocks, G, bs, D], v_cache [blocks, G, bs, Dv]) at ``slot_mapping``."""
+    if not _dev(qkv):
+        return R.unit_rms_qk_and_cache(qkv, H, G, D, Dv, eps, k_cache, v_cache, slot_mapping)
+    T = qkv.shape[0]
+    assert qkv.stride(1) == 1 and qkv.shape[1] == (H + G) * D + G * Dv
+    assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and slot_mapping.dtype == torch.int64
+    assert k_cache.shape[1:] == (G, k_cache.shape[2], D) and v_cache.shape[1:] == (G, k_cache.shape[2], Dv)
+    qn = torch.empty((T, H, D), dtype=torch.float32, device=qkv.device)
+    N.call("vda_unit_rms_qk_cache", qn.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(),
+           v_cache.data_ptr(), slot_mapping.data_ptr(), T, H, G, D, Dv, k_cache.shape[2], float(eps),
+           N.dt(qkv.dtype), N.stream())
+    return qn
+
+
+def sigmoid_window_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                             block_table: torch.Tensor, seq_lens: torch.Tensor, query_start_loc: torch.Tensor,
+                             talk: torch.Tensor, pb: torch.Tensor, scale: float, window: int, keep_first: int,
+                             max_query_len: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[i, h] = sum_j sigmoid(sum_g talk[h, g] * scale * qn[i, g] . k[j, kv(g)] + pb[h]) v[j, kv(h)] over the keys
+    j <= i with i - j < window or j < keep_first (window 0: all of them).  qn fp32 [T, H, D]; talk [H, H] and pb [H]
+    fp32; returns [T, H * Dv] in ``out_dtype`` (the cache's type)."""
+    if not _dev(qn):
+        return R.sigmoid_window_attention(qn, k_cache, v_cache, block_table, seq_lens, query_start_loc, talk, pb,
+                                          scale, window, keep_first, out_dtype)
+    T, H, D = qn.shape
+    G, bs, Dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    S = seq_lens.shape[0]
+    assert qn.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and out_dtype == k_cache.dtype
+    assert talk.dtype == torch.float32 and talk.is_contiguous() and pb.dtype == torch.float32
+    out = torch.zeros((T, H * Dv), dtype=out_dtype, device=qn.device)
+    N.call("vda_sigmoid_window_attention", out.data_ptr(), qn.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+           block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(),
+           talk.data_ptr(), pb.data_ptr(), float(scale), int(window), int(keep_first), S, H, G, D, Dv, bs,
+           max(int(max_query_len), 1), N.dt(out_dtype), N.stream())
+    return out
+
+
+# ---- gated delta rule --------------------------------------------------------------------------------------
+def gated_delta_rule(qkv: torch.Tensor, a_raw: torch.Tensor, b_raw: torch.Tensor, gate_raw: torch.Tensor,
+                     a_log: torch.Tensor, dt_bias: torch.Tensor, norm_w: torch.Tensor, state: torch.Tensor,
+                     query_start_loc: torch.Tensor, seq_lens: torch.Tensor, slot_table: torch.Tensor,
+                     H: int, G: int, D: int, Dv: int, eps: float) -> torch.Tensor:
+    """Gated delta rule with a decay per head and key channel over a ragged batch (see ops/csrc/delta_rule.hip).
+    qkv [T, 2*G*D + H*Dv] (convolved q | k | v), a_raw [T, H*D], b_raw [T, H], gate_raw [T, H*Dv] in the activation
+    type; a_log [H], dt_bias [H*D], norm_w [Dv] fp32; state fp32 [slots, H, Dv, D] (transposed), updated in place;
+    sequence s uses slot ``slot_table[s, 0]`` and starts from zero when all its tokens are in this batch."""
+    if not _dev(qkv):
+        return R.gated_delta_rule(qkv, a_raw, b_raw, gate_raw, a_log, dt_bias, norm_w, state, query_start_loc,
+                                  seq_lens, slot_table, H, G, D, Dv, eps)
+    T = qkv.shape[0]
+    S = seq_lens.shape[0]
+    for t in (qkv, a_raw, b_raw, gate_raw):
+        assert t.stride(1) == 1 and t.dtype == qkv.dtype and t.shape[0] == T
+    assert qkv.shape[1] == 2 * G * D + H * Dv and a_raw.shape[1] == H * D and b_raw.shape[1] == H
+    assert gate_raw.shape[1] == H * Dv and state.dtype == torch.float32 and state.is_contiguous()
+    assert state.shape[1:] == (H, Dv, D)
+    for t in (a_log, dt_bias, norm_w):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    out = torch.empty((T, H * Dv), dtype=qkv.dtype, device=qkv.device)
+    N.call("vda_gated_delta_rule", out.data_ptr(), out.stride(0), qkv.data_ptr(), qkv.stride(0), a_raw.data_ptr(),
+           a_raw.stride(0), b_raw.data_ptr(), b_raw.stride(0), gate_raw.data_ptr(), gate_raw.stride(0),
+           a_log.data_ptr(), dt_bias.data_ptr(), norm_w.data_ptr(), state.data_ptr(), query_start_loc.data_ptr(),
+           seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), S, H, G, D, Dv, float(eps),
+           N.dt(qkv.dtype), N.stream())
+    return out

@@ -84,16 +84,55 @@ def _compile_one(src: str, obj: str, flags: list[str], force: bool, cc: str | No
     return src, True
 
 
-def build(force: bool = False, jobs: int | None = None, verbose: bool = True) -> list[str]:
-    jobs = jobs or min(8, os.cpu_count() or 1)
+# kernels every generation path launches (linear layers, gated activations, norms, sampling); a model class adds its
+# own in ``native_sources``
+COMMON_OPS_SOURCES = ("activation.hip", "norm.hip", "sampling.hip", "gemm_dense.hip", "gemv.hip", "gemm_decode.hip")
+
+
+def ensure_built_for(model_dir: str | None, log=None) -> None:
+    """Build what a fresh checkout lacks before the engine starts.  When the model's class lists the kernel files
+    it launches (``native_sources``), only those and the common ones are compiled into libvda_ops.so (a later full
+    build adds the rest); otherwise everything is."""
+    out = log or sys.stderr
+    have = all(os.path.exists(spec["out"]) for name, spec in LIBS.items() if name != "libvda_comm.so")
+    if have:
+        return
+    only = None
+    try:
+        import json
+        with open(os.path.join(model_dir, "config.json")) as f:
+            d = json.load(f)
+        from ..config import load_hf_config
+        from ..models.registry import ModelRegistry
+        cls, _ = ModelRegistry.resolve_model_cls(list(load_hf_config(model_dir).get("architectures") or []))
+        extra = getattr(cls, "native_sources", None)
+        if extra is not None:
+            only = tuple(COMMON_OPS_SOURCES) + tuple(extra)
+    except Exception as e:       # unknown model: build everything, the engine will say what is wrong with it
+        print(f"[build] model not recognised before the build ({type(e).__name__}): building all kernels", file=out,
+              flush=True)
+    print(f"[build] native libraries missing: compiling {'all kernels' if only is None else ', '.join(only)}",
+          file=out, flush=True)
+    build(verbose=False, only=only, skip=("libvda_comm.so",) if only is not None else ())
+    print("[build] done", file=out, flush=True)
+
+
+def build(force: bool = False, jobs: int | None = None, verbose: bool = True, only: tuple | None = None,
+          skip: tuple = ()) -> list[str]:
+    """``only``: file names of ops/csrc to put into libvda_ops.so (None: all of them)."""
+    jobs = jobs or min(16, os.cpu_count() or 1)
     flags = [f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-ffast-math", "-fno-finite-math-only",
-             "-fvisibility=hidden", "-Wno-unused-value", "-DNDEBUG"]
+             "-fvisibility=hidden", "-Wno-unused-value", "-DNDEBUG",
+             # no packed fp32 arithmetic: the compiler forms v_pk_*_f32 from plain float code by itself
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     built = []
     for name, spec in LIBS.items():
         srcdir = spec["dir"]
-        if not os.path.isdir(srcdir):
+        if not os.path.isdir(srcdir) or name in skip:
             continue
         srcs = sorted(os.path.join(srcdir, f) for f in os.listdir(srcdir) if f.endswith((".hip", ".cpp")))
+        if only is not None and name == "libvda_ops.so":
+            srcs = [p_ for p_ in srcs if os.path.basename(p_) in only]
         if not srcs:
             continue
         objdir = os.path.join(HERE, "build", name.split(".")[0])
@@ -110,12 +149,18 @@ def build(force: bool = False, jobs: int | None = None, verbose: bool = True) ->
                 if verbose and did:
                     print(f"[build] compiled {os.path.relpath(src, PKG)}", flush=True)
         out = spec["out"]
-        if changed or not os.path.exists(out):
+        # a library linked from a subset of the sources is completed by the next full build
+        listing = os.path.join(objdir, "linked.txt")
+        linked = open(listing).read().split() if os.path.exists(listing) else None
+        want = sorted(os.path.basename(o) for o in objs)
+        if changed or not os.path.exists(out) or (linked is not None and linked != want):
             cmd = [cc, "-shared", "-fPIC", "-o", out, *objs, *spec["ldflags"]] if host else \
                 [_hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", out, *objs, *spec["ldflags"]]
             r = subprocess.run(cmd, capture_output=True, text=True)
             if r.returncode != 0:
                 raise RuntimeError(f"link failed for {name}:\n{r.stdout}\n{r.stderr}")
+            with open(listing, "w") as f:
+                f.write("\n".join(want))
             if verbose:
                 print(f"[build] linked {os.path.relpath(out, PKG)}", flush=True)
         built.append(out)

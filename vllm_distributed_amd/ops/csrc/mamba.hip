@@ -66,14 +66,16 @@ VDA_EXPORT int vda_causal_conv1d(void* out, const void* x, const void* weight, c
                                  int C, int W, int max_q, long x_stride, long o_stride, int act, int dtype,
                                  hipStream_t st) {
   if (S <= 0 || C <= 0) return 0;
-  if (W < 2 || W > 4) return -1;
+  if (W < 2 || W > 8) return -1;
   const int chunk = 64;
   const int nz = max(1, (max_q + chunk - 1) / chunk);
   dim3 block(256), grid((C + 255) / 256, S, nz);
 #define L(TT, WW, MODE, G) hipLaunchKernelGGL((causal_conv1d_kernel<TT, WW>), G, block, 0, st, (TT*)out, (const TT*)x, \
     (const TT*)weight, (const TT*)bias, (TT*)conv_state, qsl, seq_lens, block_table, bt_stride, C, x_stride, o_stride,  \
     act, chunk, MODE)
-#define BYW(TT, MODE, G) do { if (W == 4) L(TT, 4, MODE, G); else if (W == 3) L(TT, 3, MODE, G); else L(TT, 2, MODE, G); } while (0)
+#define BYW(TT, MODE, G) do { switch (W) { case 2: L(TT, 2, MODE, G); break; case 3: L(TT, 3, MODE, G); break; \
+    case 4: L(TT, 4, MODE, G); break; case 5: L(TT, 5, MODE, G); break; case 6: L(TT, 6, MODE, G); break;         \
+    case 7: L(TT, 7, MODE, G); break; default: L(TT, 8, MODE, G); break; } } while (0)
 #define RUN(TT) do { if (nz == 1) BYW(TT, 0, grid); else { BYW(TT, 1, grid); dim3 g2((C + 255) / 256, S, 1); BYW(TT, 2, g2); } } while (0)
   if (dtype == VDA_BF16) RUN(bf16_t);
   else if (dtype == VDA_F16) RUN(f16_t);

@@ -84,6 +84,11 @@ _SIGS = {
     "vda_lora_expand": [P, P, P, P, I, I, I, L, I, P],
     "vda_causal_conv1d": [P, P, P, P, P, P, P, P, L, I, I, I, I, L, L, I, I, P],
     "vda_lightning_decode": [P, P, P, P, P, P, L, I, I, I, L, I, P],
+    "vda_stream_embed": [P, P, P, F, I, I, I, L, I, P],
+    "vda_stream_step": [P, P, L, P, P, P, P, P, F, I, I, I, L, I, I, P],
+    "vda_unit_rms_qk_cache": [P, P, L, P, P, P, I, I, I, I, I, I, F, I, P],
+    "vda_sigmoid_window_attention": [P, P, P, P, P, L, P, P, P, P, F, I, I, I, I, I, I, I, I, I, I, P],
+    "vda_gated_delta_rule": [P, L, P, L, P, L, P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, I, F, I, P],
     "vda_selective_scan": [P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, L, L, L, L, L, L, I, I, I, I, I, I, P, P,
                            I, P],
 }
@@ -139,6 +144,10 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def call(name: str, *args) -> None:
-    rc = getattr(lib(), name)(*args)
+    fn = getattr(lib(), name, None)
+    if fn is None:
+        raise RuntimeError(f"{library_path()} has no kernel {name}: it was built from a subset of the sources; "
+                           "run `python -m vllm_distributed_amd.ops.build` to complete it")
+    rc = fn(*args)
     if rc != 0:
         raise RuntimeError(f"{name} failed with code {rc}")

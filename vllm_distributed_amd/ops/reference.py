@@ -561,3 +561,114 @@ def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale
         sc = sc.masked_fill(pos >= lim, float("-inf"))
         out[a:b] = torch.einsum("nhl,ld->nhd", torch.softmax(sc, dim=-1), V).to(q.dtype)
     return out
+
+
+# ---- residual streams (hyper-connections) ---------------------------------------------------------
+def stream_embed(ids, weight, scale: float, streams: int):
+    """fp32 residual streams [streams, T, W], every one a copy of ``weight[ids] * scale``."""
+    x = weight[ids.long()].float() * scale
+    return x.unsqueeze(0).repeat(streams, 1, 1)
+
+
+def stream_mix_norm(xs, w_in, gain, eps: float, out_dtype):
+    """h = u / sqrt(mean(u^2) + eps) * gain with u = sum_s w_in[s] xs[s]; one gain for the whole row."""
+    u = (xs.float() * w_in.float().view(-1, 1, 1)).sum(0)
+    h = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * gain.float()
+    return h.to(out_dtype)
+
+
+def stream_update(xs, y, mix, w_out):
+    """xs[t] <- sum_s mix[s, t] xs[s] + w_out[t] * y for all t at once, in place."""
+    new = torch.einsum("st,snw->tnw", mix.float(), xs.float()) + w_out.float().view(-1, 1, 1) * y.float().unsqueeze(0)
+    xs.copy_(new)
+    return xs
+
+
+# ---- sigmoid attention with mixed head scores over a window plus kept first tokens ------------------
+def unit_rms_qk_and_cache(qkv, H: int, G: int, D: int, Dv: int, eps: float, k_cache, v_cache, slot_mapping):
+    """qkv [T, H*D + G*D + G*Dv] -> q / rms(q) per head as fp32 [T, H, D]; k / rms(k) and v go to the paged cache
+    (k_cache [blocks, G, bs, D], v_cache [blocks, G, bs, Dv]) at ``slot_mapping`` (negative: not stored)."""
+    T = qkv.shape[0]
+    q = qkv[:, : H * D].float().view(T, H, D)
+    k = qkv[:, H * D: (H + G) * D].float().view(T, G, D)
+    v = qkv[:, (H + G) * D:].view(T, G, Dv)
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+    if k_cache is not None:
+        bs = k_cache.shape[2]
+        ok = slot_mapping[:T] >= 0
+        sl = slot_mapping[:T][ok].long()
+        k_cache[sl // bs, :, sl % bs] = k[ok].to(k_cache.dtype)
+        v_cache[sl // bs, :, sl % bs] = v[ok].to(v_cache.dtype)
+    return q
+
+
+def sigmoid_window_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, talk, pb, scale: float, window: int,
+                             keep_first: int, out_dtype):
+    """Per sequence: raw[g, i, j] = scale * qn[i, g] . k[j, kv(g)]; mixed[h] = sum_g talk[h, g] raw[g];
+    weight = sigmoid(mixed + pb[h]) on the visible keys (j <= i and (i - j < window or j < keep_first); window 0 =
+    every earlier key), no normalisation over keys; out[i, h] = sum_j weight[h, i, j] v[j, kv(h)]."""
+    T, H, D = qn.shape
+    G, bs, Dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    out = torch.zeros((T, H, Dv), dtype=torch.float32, device=qn.device)
+    rep = H // G
+    for s in range(seq_lens.shape[0]):
+        sl = int(seq_lens[s])
+        t0, t1 = int(qsl[s]), int(qsl[s + 1])
+        L = t1 - t0
+        if sl <= 0 or L <= 0:
+            continue
+        nb = -(-sl // bs)
+        blocks = block_table[s, :nb].long()
+        k = k_cache[blocks].float().permute(0, 2, 1, 3).reshape(nb * bs, G, D)[:sl]
+        v = v_cache[blocks].float().permute(0, 2, 1, 3).reshape(nb * bs, G, Dv)[:sl]
+        kk, vv = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
+        raw = torch.einsum("ihd,jhd->hij", qn[t0:t1].float(), kk) * scale
+        mixed = torch.einsum("hg,gij->hij", talk.float(), raw)
+        i = torch.arange(sl - L, sl, device=qn.device)[:, None]
+        j = torch.arange(sl, device=qn.device)[None, :]
+        vis = j <= i
+        if window > 0:
+            vis = vis & ((i - j < window) | (j < keep_first))
+        w = torch.sigmoid(mixed + pb.float().view(-1, 1, 1)) * vis
+        out[t0:t1] = torch.einsum("hij,jhd->ihd", w, vv)
+    return out.view(T, H * Dv).to(out_dtype)
+
+
+# ---- gated delta rule with one decay per key channel ---------------------------------------------------
+def gated_delta_rule(qkv, a_raw, b_raw, gate_raw, a_log, dt_bias, norm_w, state, qsl, seq_lens, slot_table,
+                     H: int, G: int, D: int, Dv: int, eps: float):
+    """qkv [T, 2*G*D + H*Dv] (after the short convolution), a_raw [T, H*D], b_raw [T, H], gate_raw [T, H*Dv];
+    state fp32 [slots, H, Dv, D] (S transposed), updated in place.  Per token and head (q, k of head h // (H / G)):
+    q <- q / sqrt(|q|^2 + 1e-6) / sqrt(D), k <- k / sqrt(|k|^2 + 1e-6), decay = exp(-exp(a_log[h]) *
+    softplus(a_raw + dt_bias)); S <- decay[:, None] * S; u = sigmoid(b) * (v - S^T k); S <- S + k u^T; o = S^T q;
+    out = o / rms(o) * norm_w * sigmoid(gate_raw)."""
+    T = qkv.shape[0]
+    out = torch.zeros((T, H, Dv), dtype=torch.float32, device=qkv.device)
+    rep = H // G
+    q = qkv[:, : G * D].float().view(T, G, D)
+    k = qkv[:, G * D: 2 * G * D].float().view(T, G, D)
+    v = qkv[:, 2 * G * D:].float().view(T, H, Dv)
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+    q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(b_raw.float())
+    decay = torch.exp(-torch.exp(a_log.float()).view(1, H, 1)
+                      * torch.nn.functional.softplus(a_raw.float() + dt_bias.float()).view(T, H, D))
+    for s in range(seq_lens.shape[0]):
+        sl = int(seq_lens[s])
+        t0, t1 = int(qsl[s]), int(qsl[s + 1])
+        if sl <= 0 or t1 <= t0:
+            continue
+        slot = int(slot_table[s, 0])
+        S = state[slot].transpose(1, 2).clone() if sl - (t1 - t0) > 0 else \
+            torch.zeros((H, D, Dv), dtype=torch.float32, device=qkv.device)
+        for t in range(t0, t1):
+            S = decay[t].unsqueeze(-1) * S
+            u = beta[t].unsqueeze(-1) * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+            S = S + k[t].unsqueeze(-1) * u.unsqueeze(1)
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S.transpose(1, 2)
+    o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    o = o * torch.sigmoid(gate_raw.float().view(T, H, Dv))
+    return o.view(T, H * Dv).to(qkv.dtype)

@@ -52,6 +52,20 @@ class AttentionSpec(KVCacheSpec):
 @dataclass(frozen=True)
 class FullAttentionSpec(AttentionSpec):
     sliding_window: Optional[int] = None   # kept so hybrid models can be served with one group
+    # values narrower or wider than keys (None: the key width); the V tensor then has its own size
+    v_head_size: Optional[int] = None
+    # V stored [blocks, kv_heads, block, width] like K, instead of the MFMA kernels' [blocks, kv_heads, width, block]
+    token_major_v: bool = False
+
+    @property
+    def k_bytes_per_block(self) -> int:
+        return self.block_size * self.num_kv_heads * self.head_size * _dtype_size(self.dtype)
+
+    @property
+    def page_size_bytes(self) -> int:
+        if self.v_head_size is None:
+            return super().page_size_bytes
+        return self.block_size * self.num_kv_heads * (self.head_size + self.v_head_size) * _dtype_size(self.dtype)
 
     @property
     def type_id(self) -> str:

@@ -74,6 +74,11 @@ class SchedulerOutput:
     tknp: Optional[TokenParallelAllocation] = None
     # run-ahead scheduling: the runner may hand back a handle and leave the sampled ids on the device until asked
     defer_output: bool = False
+    # requests whose next tokens are given from outside (replay of a recorded run, teacher forcing): the runner
+    # discards what it samples for them
+    forced_req_ids: set[str] = field(default_factory=set)
+    # request -> indices among the tokens it runs in this step whose full-vocabulary logits are returned
+    logit_taps: dict[str, list[int]] = field(default_factory=dict)
 
 
 @dataclass
@@ -91,6 +96,8 @@ class ModelRunnerOutput:
     # subset of finished_recving whose transfer failed: nothing usable arrived, the prompt is computed locally
     failed_recving: Optional[set[str]] = None
     num_nans_in_logits: Optional[dict[str, int]] = None
+    # request -> fp32 logits [taps, vocab] (host) for the step's ``logit_taps``
+    tapped_logits: dict[str, Any] = field(default_factory=dict)
 
 
 EMPTY_MODEL_RUNNER_OUTPUT = ModelRunnerOutput()

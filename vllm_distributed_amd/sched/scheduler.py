@@ -134,13 +134,17 @@ class Scheduler(SchedulerInterface):
         self.encoder_cache_manager = EncoderCacheManager(sc.encoder_cache_size)
         self.max_num_encoder_input_tokens = sc.max_num_encoder_input_tokens
         self._step = 0
+        # requests that are fed their next tokens from outside (extend_request) instead of sampling them
+        self.forced: set[str] = set()
         self.async_mode = bool(self.scheduler_config.async_scheduling)
         self.last_schedule_preempted = False
 
     # ------------------------------------------------------------------
     # schedule
     # ------------------------------------------------------------------
-    def schedule(self) -> SchedulerOutput:
+    def schedule(self, plan: Optional[dict[str, int]] = None) -> SchedulerOutput:
+        """``plan`` (replay of a recorded run): only the named requests run in this step, each exactly the given
+        number of its known tokens; admission, block allocation and batching are the ordinary ones."""
         new_reqs: list[Request] = []
         resumed_reqs: list[Request] = []
         running_reqs: list[Request] = []
@@ -166,6 +170,14 @@ class Scheduler(SchedulerInterface):
             thr = self.scheduler_config.long_prefill_token_threshold
             if 0 < thr < n_new:
                 n_new = thr
+            if plan is not None:
+                if req.request_id not in plan:
+                    i += 1
+                    continue
+                if not 0 < plan[req.request_id] <= min(n_new, budget):
+                    raise ValueError(f"the plan gives request {req.request_id} {plan[req.request_id]} tokens, "
+                                     f"{min(n_new, budget)} can run")
+                n_new = plan[req.request_id]
             n_new = min(n_new, budget, self.max_model_len - 1 - req.num_computed_tokens)
             enc_ids, n_new, new_enc_budget = self._schedule_encoder(req, req.num_computed_tokens, n_new,
                                                                    encoder_budget)
@@ -242,6 +254,10 @@ class Scheduler(SchedulerInterface):
                 if len(self.running) >= self.max_num_running_reqs:
                     break
                 req = self.waiting.peek_request()
+                if plan is not None and req.request_id not in plan:
+                    self.waiting.pop_request()
+                    skipped.prepend_request(req)
+                    continue
 
                 if req.status == RequestStatus.WAITING_FOR_REMOTE_KVS:
                     if not self._update_waiting_for_remote_kv(req):
@@ -292,6 +308,11 @@ class Scheduler(SchedulerInterface):
                         skipped.prepend_request(req)
                         continue
                     n_new = min(n_new, budget)
+                    if plan is not None:
+                        if not 0 < plan[req.request_id] <= n_new:
+                            raise ValueError(f"the plan gives request {req.request_id} {plan[req.request_id]} "
+                                             f"tokens, {n_new} can run")
+                        n_new = plan[req.request_id]
                     assert n_new > 0
                     enc_ids, n_new, new_enc_budget = self._schedule_encoder(req, n_computed, n_new,
                                                                            encoder_budget)
@@ -372,6 +393,8 @@ class Scheduler(SchedulerInterface):
             finished_req_ids=self.finished_req_ids,
             free_encoder_input_ids=self.encoder_cache_manager.get_freed_ids(),
             structured_output_request_ids=structured_ids, grammar_bitmask=bitmask)
+        if self.forced:
+            out.forced_req_ids = {rid for rid in num_scheduled if rid in self.forced}
         if tknp is not None:
             out.tknp = tknp.allocation(num_scheduled)
         if self.connector is not None:
@@ -448,8 +471,9 @@ class Scheduler(SchedulerInterface):
             rid = req.request_id
             d.req_ids.append(rid)
             d.resumed_from_preemption.append(resumed)
-            if use_pp or resumed:
-                # first-stage workers never see sampled tokens: ship the ones this step consumes
+            if use_pp or resumed or rid in self.forced:
+                # first-stage workers never see sampled tokens (and nobody has seen tokens given from outside):
+                # ship the ones this step consumes
                 n_tok = num_scheduled[rid] - len(spec_tokens.get(rid, ()))
                 s = req.num_computed_tokens
                 d.new_token_ids.append(list(req.all_token_ids[s:s + n_tok]))
@@ -586,11 +610,22 @@ class Scheduler(SchedulerInterface):
     # ------------------------------------------------------------------
     # request lifecycle
     # ------------------------------------------------------------------
-    def add_request(self, request: Request) -> None:
+    def add_request(self, request: Request, forced: bool = False) -> None:
+        """``forced``: the request's continuation will be given with ``extend_request``; nothing sampled is kept."""
         self.waiting.add_request(request)
         self.requests[request.request_id] = request
+        if forced:
+            self.forced.add(request.request_id)
         if self.log_stats:
             request.record_event(EngineCoreEventType.QUEUED)
+
+    def extend_request(self, request_id: str, token_ids: list[int]) -> None:
+        """Append tokens given from outside to a live request (replay of a recorded run, teacher forcing).  From
+        its first extension on the request no longer takes sampled tokens; the workers receive the new tokens with
+        the step that runs them."""
+        req = self.requests[request_id]
+        self.forced.add(request_id)
+        req.append_output_token_ids(list(token_ids))
 
     def finish_requests(self, request_ids: Union[str, Iterable[str]], finished_status: RequestStatus) -> None:
         assert RequestStatus.is_finished(finished_status)
@@ -620,6 +655,7 @@ class Scheduler(SchedulerInterface):
         delay = delay or keep_blocks
         self.encoder_cache_manager.free(req)
         rid = req.request_id
+        self.forced.discard(rid)
         self.finished_req_ids.add(rid)
         if self.finished_req_ids_dict is not None:
             self.finished_req_ids_dict[req.client_index].add(rid)

@@ -238,7 +238,8 @@ class ModelRunner:
         # every layer that owns per-request cache memory: attention layers and state-space mixers
         self.attn_layers = {n: m for n, m in self.model.named_modules()
                             if (isinstance(m, Attention) or getattr(m, "is_state_space_layer", False)
-                                or getattr(m, "is_mla", False)) and getattr(m, "kv_source", None) is None}
+                                or getattr(m, "is_mla", False) or getattr(m, "is_paged_kv_layer", False))
+                            and getattr(m, "kv_source", None) is None}
         for n, m in self.attn_layers.items():
             m.layer_name = n
         # heads of a size the kernels do not have run zero-padded (layers/attention.py): size buffers for that
@@ -416,7 +417,7 @@ class ModelRunner:
         row of the persistent batch + 1; slot 0 absorbs the padding rows of captured decode graphs."""
         self.state_table: Optional[torch.Tensor] = None
         ss = {n: m for n, m in self.attn_layers.items() if getattr(m, "is_state_space_layer", False)}
-        if not ss or len(ss) == len(self.attn_layers):
+        if not ss or (len(ss) == len(self.attn_layers) and not getattr(self.model, "row_state_slots", False)):
             return
         nslots = max(self.max_num_reqs, max(self.capture_sizes, default=0)) + 1
         total = 0
@@ -561,12 +562,19 @@ class ModelRunner:
                     off += t.size
                     continue
                 half = t.size // 2
+                vd = getattr(sp, "v_head_size", None) or sp.head_size
+                if vd != sp.head_size:                 # keys and values of different widths
+                    half = nb * sp.k_bytes_per_block
                 k = raw[:half].view(sp.dtype).view(nb, sp.num_kv_heads, sp.block_size, sp.head_size)
-                v = raw[half:].view(sp.dtype).view(nb, sp.num_kv_heads, sp.head_size, sp.block_size)
+                if getattr(sp, "token_major_v", False):
+                    v = raw[half:].view(sp.dtype).view(nb, sp.num_kv_heads, sp.block_size, vd)
+                else:
+                    v = raw[half:].view(sp.dtype).view(nb, sp.num_kv_heads, vd, sp.block_size)
                 for n in t.shared_by:
                     self.attn_layers[n].bind_kv_cache(k, v)
                     self.kv_layer_loc[n] = (ci, off, half)
-                    self.kv_layer_parts[n] = [(ci, off, half, sp.num_kv_heads), (ci, off + half, half, sp.num_kv_heads)]
+                    self.kv_layer_parts[n] = [(ci, off, half, sp.num_kv_heads),
+                                              (ci, off + half, t.size - half, sp.num_kv_heads)]
                 self.kv_caches.append((k, v))
                 off += t.size
         self.input_batch = InputBatch(self.max_num_reqs, self.max_model_len, self.block_size, self.vocab_size,
@@ -1136,9 +1144,11 @@ class ModelRunner:
         else:
             sampled_lists = [[t] for t in sampled_t.tolist()]
         self._check_comm_errors()            # the stream is drained: a timed-out collective has reported by now
-        # requests still in the middle of their prompt discard the sample
+        # requests still in the middle of their prompt discard the sample, and so do requests whose next tokens
+        # are given from outside
+        forced = so.forced_req_ids
         for i in range(len(req_ids)):
-            if not done[i]:
+            if not done[i] or (forced and req_ids[i] in forced):
                 sampled_lists[i] = []
         self._apply_sampled(req_ids, sampled_lists)
         spec_tokens = None
@@ -1152,6 +1162,8 @@ class ModelRunner:
             prompt_logprobs_dict=prompt_lp, finished_sending=finished_sending, finished_recving=finished_recving,
             failed_recving=failed_recving,
             num_nans_in_logits=getattr(self, "_last_nans", None))
+        if so.logit_taps:
+            result.tapped_logits = self._tap_logits(so, hidden, req_ids, n_sched, cu)
         if tmd is not None and not tk_plain:
             get_tknp_group().broadcast_object(result, src=0)
         return result
@@ -1344,6 +1356,23 @@ class ModelRunner:
             ids, lps, ranks = Sampler.gather_logprobs(lp, k, tgt)
             out[rid] = LogprobsLists(ids.tolist(), lps.tolist(), ranks.tolist())
         return out
+
+    def _tap_logits(self, so, hidden, req_ids, n_sched, cu) -> dict:
+        """Full-vocabulary fp32 logits at the positions ``so.logit_taps`` names, per request, on the host."""
+        idx, spans = [], {}
+        for i, rid in enumerate(req_ids):
+            taps = so.logit_taps.get(rid)
+            if not taps:
+                continue
+            if min(taps) < 0 or max(taps) >= int(n_sched[i]):
+                raise ValueError(f"logit taps {taps} of request {rid} lie outside its {int(n_sched[i])} tokens")
+            spans[rid] = (len(idx), len(idx) + len(taps))
+            idx.extend(int(cu[i]) + int(t) for t in taps)
+        if not idx:
+            return {}
+        sel = torch.tensor(idx, dtype=torch.int64, device=self.device)
+        logits = self._compute_logits(hidden[sel], np.asarray(idx)).float().cpu().numpy()
+        return {rid: logits[a:b] for rid, (a, b) in spans.items()}
 
     def _compute_logits(self, hidden_rows: torch.Tensor, index: np.ndarray) -> torch.Tensor:
         """Logits of rows ``index`` of this step's tokens (the index tells LoRA which adapter each row uses)."""
