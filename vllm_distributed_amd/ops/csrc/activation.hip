@@ -108,6 +108,8 @@ VDA_EXPORT int vda_act_and_mul(void* out, const void* in, long rows, int d, long
     return launch_gated<bf16_t>(out, in, rows, d, in_stride, out_stride, act_kind, act_first, threshold, fp8_scale, st);
   if (dtype == VDA_F16)
     return launch_gated<f16_t>(out, in, rows, d, in_stride, out_stride, act_kind, act_first, threshold, fp8_scale, st);
+  if (dtype == VDA_F32)
+    return launch_gated<float>(out, in, rows, d, in_stride, out_stride, act_kind, act_first, threshold, fp8_scale, st);
   return -3;
 }
 

@@ -18,6 +18,7 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -25,6 +26,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 template <typename T> struct Vec;
 template <> struct Vec<bf16_t> { using v8 = bf16x8; using v4 = bf16x4; };
 template <> struct Vec<f16_t> { using v8 = f16x8; using v4 = f16x4; };
+template <> struct Vec<float> { using v8 = f32x8; using v4 = f32x4; };      // fp32 activations (elementwise kernels)
 
 template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }

@@ -69,6 +69,10 @@ class FullAttentionSpec(AttentionSpec):
 
     @property
     def type_id(self) -> str:
+        if self.v_head_size is not None or self.token_major_v:
+            # equal page bytes do not make equal tensors here: the split between K and V is part of the type
+            return (f"full_{self.block_size}_{self.num_kv_heads}x{self.head_size}+{self.v_head_size or self.head_size}"
+                    f"{'t' if self.token_major_v else ''}_{_dtype_size(self.dtype)}")
         return f"full_{self.block_size}_{self.page_size_bytes}"
 
     def max_memory_usage_bytes(self, max_model_len: int, max_num_batched_tokens: int) -> int:

@@ -330,7 +330,8 @@ class KVCacheManager:
         # becomes full and must be hashed).  While a step stays below both marks allocate_slots returns at once.
         # Only for layouts whose every group is plain full attention (windows release blocks as they go).
         self._covered: dict[str, tuple[int, int]] = {}
-        self._fast_ok = all(type(m) is FullAttentionManager for m in self.coordinator.managers)
+        self._fast_ok = bool(self.coordinator.managers) and all(type(m) is FullAttentionManager
+                                                                 for m in self.coordinator.managers)
         self._no_blocks = self._empty()
 
     @property

@@ -162,7 +162,10 @@ def _num_blocks(vllm_config, available: int, page_size: int, num_layers: int) ->
 def get_kv_cache_config(vllm_config, spec: dict[str, KVCacheSpec], available: int) -> KVCacheConfig:
     """Turn a per-layer spec + a byte budget into tensors, groups and a block count."""
     if not spec:
-        return KVCacheConfig(num_blocks=1, kv_cache_tensors=[], kv_cache_groups=[])
+        # no layer keeps pages (every mixer holds its state in the runner's per-row slots): the pool is only the
+        # scheduler's book-keeping
+        nb = max(2, int(vllm_config.cache_config.num_gpu_blocks_override or 2))
+        return KVCacheConfig(num_blocks=nb, kv_cache_tensors=[], kv_cache_groups=[])
     if vllm_config.cache_config.num_gpu_blocks_override is None:
         _check_enough_memory(vllm_config, spec, available)
     if not _uniform_type(spec):
