@@ -625,6 +625,7 @@ def dense_gemm_wanted(x: torch.Tensor, w: torch.Tensor, max_n: Optional[int] = N
     batches stay on the library GEMM."""
     return (x.is_cuda and envs.VDA_DENSE_GEMM_MIN_M <= x.shape[0] <= envs.VDA_DENSE_GEMM_MAX_M
             and 64 <= w.shape[0] <= (envs.VDA_DENSE_GEMM_MAX_N if max_n is None else max_n)
+            and w.shape[0] % 4 == 0          # the kernel stores (and splits K over) groups of four output columns
             and dense_gemm_ok(x, w) and w.shape[1] == x.shape[1])
 
 
