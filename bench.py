@@ -139,6 +139,11 @@ def main() -> None:
                     help="disaggregated prefill/decode instead of the flagship run: e.g. 1p1d or 4p4d, Llama-3-8B, "
                          "1024-token prompts, 200 generated tokens (benchmarks/disagg.py); needs x + y GPUs unless "
                          "--rehearse-on-one-gpu")
+    ap.add_argument("--compare-nositar", action="store_true",
+                    help="instead of the flagship run: prefill / decode throughput of Nositar stacks beside a "
+                         "sliding-window Llama and a Jamba stack of equal size (benchmarks/hybrid_compare.py; "
+                         "--batch / --input-len / --output-len apply, one JSON line per model and size)")
+    ap.add_argument("--sizes", default="small,medium", help="--compare-nositar: small, medium, large")
     ap.add_argument("--rehearse-on-one-gpu", action="store_true", help="--disagg: every engine on GPU 0")
     ap.add_argument("--kv-push", action="store_true", help="--disagg: push blocks while prefilling (landing pool)")
     ap.add_argument("--num-prompts", type=int, default=200, help="--disagg: requests")
@@ -146,6 +151,13 @@ def main() -> None:
     a = ap.parse_args()
     if a.disagg:
         return run_disagg(a)
+    if a.compare_nositar:
+        from vllm_distributed_amd.benchmarks import hybrid_compare
+        argv = ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
+                "--input-len", str(2048 if a.input_len == 1024 else a.input_len),
+                "--output-len", str(64 if a.output_len == 128 else a.output_len)]
+        hybrid_compare.main(argv + (["--enforce-eager"] if a.enforce_eager else []))
+        return
     if a.pp < 1 or a.gpus % a.pp:
         raise SystemExit(f"--pp {a.pp} does not divide --gpus {a.gpus}")
     launched = "WORLD_SIZE" in os.environ

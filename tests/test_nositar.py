@@ -119,7 +119,7 @@ def test_sigmoid_attention_paged(dev, H, G, D, E, window, keep):
     nblk = sum(-(-n // bs) for n in lens) + 3
     perm = torch.randperm(nblk - 1) + 1
     kc = torch.zeros(nblk, G, bs, D, device=dev)
-    vc = torch.zeros(nblk, G, bs, E, device=dev)
+    vc = torch.zeros(nblk, G, E, bs, device=dev)
     table = torch.zeros(len(lens), max(-(-n // bs) for n in lens), dtype=torch.int32)
     o = 0
     for s, n in enumerate(lens):
@@ -145,6 +145,52 @@ def test_sigmoid_attention_paged(dev, H, G, D, E, window, keep):
         want = O.sigmoid_attention(seqs[s], eye[: H * D], eye[H * D: (H + G) * D], eye[(H + G) * D:],
                                    torch.eye(H * E), talk, pb, H, G, D, E, scale, window, keep, eps)[n - m:]
         torch.testing.assert_close(out[o:o + m], want, atol=2e-5, rtol=2e-5)
+        o += m
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,E,window,keep,bs", [(8, 2, 48, 48, 72, 6, 16), (16, 4, 64, 64, 40, 3, 16),
+                                                    (4, 4, 128, 128, None, 0, 32), (16, 16, 32, 104, 300, 2, 16),
+                                                    (3, 1, 24, 8, 33, 40, 8)])
+def test_sigmoid_attention_matrix_core_form(monkeypatch, H, G, D, E, window, keep, bs):
+    """The 16-bit form (q.k and weights.v on the matrix cores) against the dense oracle fed with the same bf16
+    numbers, and against the plain fp32-arithmetic form of the same kernel family."""
+    from vllm_distributed_amd import envs
+    eps, scale = 1e-5, D ** -0.5
+    lens, news = [150, 333, 40, 129], [1, 70, 40, 17]
+    C = H * D + G * D + G * E
+    seqs = [torch.randn(n, C).bfloat16() for n in lens]
+    talk, pb = torch.eye(H) + 0.3 * torch.randn(H, H), torch.randn(H) - 2.0
+    nblk = sum(-(-n // bs) for n in lens) + 2
+    perm = torch.randperm(nblk - 1) + 1
+    table = torch.zeros(len(lens), max(-(-n // bs) for n in lens), dtype=torch.int32)
+    o = 0
+    for s, n in enumerate(lens):
+        k = -(-n // bs)
+        table[s, :k] = perm[o:o + k].int()
+        o += k
+    outs = {}
+    for form in ("mfma", "plain"):
+        monkeypatch.setattr(envs, "VDA_SIGMOID_ATTN_FORM", form, raising=False)
+        kc = torch.zeros(nblk, G, bs, D, device="cuda", dtype=torch.bfloat16)
+        vc = torch.zeros(nblk, G, E, bs, device="cuda", dtype=torch.bfloat16)
+        slots = torch.tensor([int(table[s, p // bs]) * bs + p % bs for s, n in enumerate(lens) for p in range(n)])
+        qn_all = ops.unit_rms_qk_and_cache(torch.cat(seqs).cuda(), H, G, D, E, eps, kc, vc, slots.cuda())
+        starts = torch.tensor([0] + lens).cumsum(0)
+        qn = torch.cat([qn_all[starts[s] + n - m: starts[s] + n] for s, (n, m) in enumerate(zip(lens, news))])
+        qsl = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32)
+        outs[form] = ops.sigmoid_window_attention(qn.contiguous(), kc, vc, table.cuda(),
+                                                  torch.tensor(lens, dtype=torch.int32).cuda(), qsl.cuda(), talk.cuda(),
+                                                  pb.cuda(), scale, window or 0, keep, max(news), torch.bfloat16
+                                                  ).float().cpu()
+    eye = torch.eye(C)
+    o = 0
+    for s, (n, m) in enumerate(zip(lens, news)):
+        want = O.sigmoid_attention(seqs[s].float(), eye[: H * D], eye[H * D: (H + G) * D], eye[(H + G) * D:],
+                                   torch.eye(H * E), talk, pb, H, G, D, E, scale, window, keep, eps)[n - m:]
+        for form in outs:      # weights are not normalised over keys: errors scale with the largest output
+            err = (outs[form][o:o + m] - want).abs().max() / want.abs().max()
+            assert err < 2e-2, f"{form}: sequence {s} differs by {err:.3f} of the largest output"
         o += m
 
 

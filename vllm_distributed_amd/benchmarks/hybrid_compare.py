@@ -1,0 +1,137 @@
+"""Prefill and decode throughput of a Nositar stack beside the closest existing models of equal size, random weights.
+
+    python bench.py --compare-nositar [--sizes small,medium] [--batch 32] [--input-len 2048] [--output-len 64]
+
+Per size three engines run one after the other, each in a process of its own (``--one`` is the child's entry):
+  nositar      alternating sigmoid head-mixing attention (window + kept first tokens) and gated delta-rule layers,
+               two residual streams, ReLU-gated feed-forward
+  llama-swa    a Llama stack of the same width, depth, heads and feed-forward with the same sliding window (the
+               framework's softmax attention kernels)
+  jamba        the framework's attention + recurrent (Mamba) hybrid of the same width, depth and feed-forward
+Prefill: ``batch`` prompts of ``input-len`` tokens, one generated token.  Decode: the same requests generating
+``output-len`` tokens, the prefill time taken off.  One JSON line per (size, model).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import subprocess
+import sys
+import tempfile
+import time
+
+SIZES = {
+    # width, layers, heads, kv heads, head dim, feed-forward, window, vocab
+    "small": dict(width=1024, layers=8, heads=16, kv_heads=4, dim=64, ff=4096, window=512, vocab=32000),
+    "medium": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=8192, window=1024, vocab=32000),
+    "large": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, ff=14336, window=1024, vocab=32000),
+}
+
+
+def nositar_config(s: dict) -> dict:
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": s["ff"]},
+           "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"],
+                     "scale": s["dim"] ** -0.5, "mask": {"size": s["window"], "keep_first": 4}}}
+    dh = max(s["width"] // 128, 1)
+    delta = {"type": "channel_delta", "mlp": {"kind": "dense", "ff": s["ff"]},
+             "mixer": {"heads": dh, "kv_heads": dh, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64,
+                       "gate_rank": 64}}
+    return {"architecture": "Nositar", "vocab": s["vocab"], "width": s["width"], "streams": 2, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+            "layers": [att if i % 2 == 0 else delta for i in range(s["layers"])]}
+
+
+def llama_config(s: dict) -> dict:
+    return {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "hidden_size": s["width"],
+            "intermediate_size": s["ff"], "num_hidden_layers": s["layers"], "num_attention_heads": s["heads"],
+            "num_key_value_heads": s["kv_heads"], "head_dim": s["dim"], "vocab_size": s["vocab"],
+            "sliding_window": s["window"], "max_position_embeddings": 32768, "rms_norm_eps": 1e-6,
+            "rope_theta": 10000.0, "tie_word_embeddings": False, "torch_dtype": "bfloat16"}
+
+
+def jamba_config(s: dict) -> dict:
+    return {"architectures": ["JambaForCausalLM"], "model_type": "jamba", "hidden_size": s["width"],
+            "intermediate_size": s["ff"], "num_hidden_layers": s["layers"], "num_attention_heads": s["heads"],
+            "num_key_value_heads": s["kv_heads"], "vocab_size": s["vocab"], "attn_layer_period": 2,
+            "attn_layer_offset": 0, "expert_layer_period": 2, "expert_layer_offset": 1, "num_experts": 1,
+            "num_experts_per_tok": 1, "mamba_expand": 2, "mamba_d_state": 16, "mamba_d_conv": 4,
+            "mamba_dt_rank": max(s["width"] // 16, 1), "mamba_proj_bias": False, "mamba_conv_bias": True,
+            "rms_norm_eps": 1e-6, "max_position_embeddings": 32768, "tie_word_embeddings": False,
+            "torch_dtype": "bfloat16"}
+
+
+MODELS = {"nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config}
+
+
+def run_one(kind: str, size: str, batch: int, input_len: int, output_len: int, eager: bool) -> dict:
+    import torch
+    from vllm_distributed_amd import LLM, SamplingParams
+    folder = tempfile.mkdtemp(prefix=f"vda_cmp_{kind}_")
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(MODELS[kind](SIZES[size]), f)
+    llm = LLM(model=folder, load_format="dummy", skip_tokenizer_init=True, dtype="bfloat16",
+              max_model_len=input_len + output_len + 16, max_num_seqs=max(batch, 8),
+              max_num_batched_tokens=16384, enable_prefix_caching=False, gpu_memory_utilization=0.6,
+              enforce_eager=eager, seed=0)
+    vocab = SIZES[size]["vocab"]
+
+    def prompts(seed):
+        g = torch.Generator().manual_seed(seed)
+        return torch.randint(10, vocab - 10, (batch, input_len), generator=g).tolist()
+
+    def timed(seed, new_tokens):
+        sp = SamplingParams(temperature=0.0, max_tokens=new_tokens, ignore_eos=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        llm.generate(prompt_token_ids=prompts(seed), sampling_params=sp)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+    timed(1, 2)                                    # warm-up: allocations, library heuristics
+    t_pre = min(timed(2, 1), timed(3, 1))
+    t_all = min(timed(4, output_len), timed(5, output_len))
+    llm.shutdown()
+    t_dec = max(t_all - t_pre, 1e-9)
+    return {"model": kind, "size": size, **{k: SIZES[size][k] for k in ("width", "layers", "heads", "dim", "window")},
+            "batch": batch, "input_len": input_len, "output_len": output_len,
+            "prefill_tokens_per_s": round(batch * input_len / t_pre, 1),
+            "decode_tokens_per_s": round(batch * (output_len - 1) / t_dec, 1),
+            "prefill_s": round(t_pre, 4), "decode_s": round(t_dec, 4), "dtype": "bf16",
+            "data": "synthetic random token prompts, random-init weights", "decode_graphs": not eager}
+
+
+def main(argv=None) -> list[dict]:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--sizes", default="small,medium")
+    ap.add_argument("--models", default="nositar,llama-swa,jamba")
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--input-len", type=int, default=2048)
+    ap.add_argument("--output-len", type=int, default=64)
+    ap.add_argument("--enforce-eager", action="store_true")
+    ap.add_argument("--one", default=None, help="internal: run one (model, size) in this process")
+    a = ap.parse_args(argv)
+    if a.one:
+        kind, size = a.one.split(":")
+        print(json.dumps(run_one(kind, size, a.batch, a.input_len, a.output_len, a.enforce_eager)), flush=True)
+        return []
+    rows = []
+    for size in a.sizes.split(","):
+        for kind in a.models.split(","):
+            cmd = [sys.executable, "-m", "vllm_distributed_amd.benchmarks.hybrid_compare", "--one", f"{kind}:{size}",
+                   "--batch", str(a.batch), "--input-len", str(a.input_len), "--output-len", str(a.output_len)]
+            if a.enforce_eager:
+                cmd.append("--enforce-eager")
+            print(f"[compare] {kind} {size} ...", file=sys.stderr, flush=True)
+            r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=900)
+            line = next((ln for ln in reversed(r.stdout.splitlines()) if ln.startswith("{")), None)
+            if r.returncode != 0 or line is None:
+                row = {"model": kind, "size": size, "error": f"exit code {r.returncode}"}
+            else:
+                row = json.loads(line)
+            rows.append(row)
+            print(json.dumps(row), flush=True)
+    return rows
+
+
+if __name__ == "__main__":
+    main()

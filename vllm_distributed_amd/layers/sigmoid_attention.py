@@ -8,8 +8,8 @@
 
 The layer owns pages of the ordinary paged KV cache (the scheduler and KV-cache manager treat it as a full-attention
 layer: kept first tokens stay in their pages at their true positions, the kernel skips what the window hides).
-Its cache keeps the NORMALISED keys, and values token-major ([blocks, kv_heads, block, vdim]); key and value widths
-may differ.  Kernels: ops/csrc/sigmoid_attention.hip.
+Its cache keeps the NORMALISED keys; the layout is the framework's (K [blocks, kv_heads, block, dim], V [blocks,
+kv_heads, vdim, block]) with key and value widths of their own.  Kernels: ops/csrc/sigmoid_attention.hip.
 """
 from __future__ import annotations
 
@@ -54,7 +54,7 @@ class SigmoidWindowAttention(nn.Module):
 
     def get_kv_cache_spec(self, block_size: int, dtype: torch.dtype) -> KVCacheSpec:
         return FullAttentionSpec(block_size=block_size, num_kv_heads=self.num_kv_heads, head_size=self.head_dim,
-                                 dtype=dtype, v_head_size=self.v_head_dim, token_major_v=True)
+                                 dtype=dtype, v_head_size=self.v_head_dim)
 
     def bind_kv_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
         self.k_cache, self.v_cache = k_cache, v_cache

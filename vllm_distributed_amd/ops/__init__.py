@@ -1297,15 +1297,15 @@ def stream_step(xs: torch.Tensor, y: Optional[torch.Tensor] = None, mix: Optiona
 def unit_rms_qk_and_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, eps: float,
                           k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                           slot_mapping: torch.Tensor) -> torch.Tensor:
-    """qkv [T, H*D + G*D + G*Dv]: returns q / rms(q) per head (fp32 [T, H, D]) and stores k / rms(k) and v in the
-    paged cache (k_cache [blocks, G, bs, D], v_cache [blocks, G, bs, Dv]) at ``slot_mapping``."""
+    """qkv [T, H*D + G*D + G*Dv]: returns q / rms(q) per head ([T, H, D], qkv's type) and stores k / rms(k) and v in the
+    paged cache (k_cache [blocks, G, bs, D], v_cache [blocks, G, Dv, bs]) at ``slot_mapping``."""
     if not _dev(qkv):
         return R.unit_rms_qk_and_cache(qkv, H, G, D, Dv, eps, k_cache, v_cache, slot_mapping)
     T = qkv.shape[0]
     assert qkv.stride(1) == 1 and qkv.shape[1] == (H + G) * D + G * Dv
     assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and slot_mapping.dtype == torch.int64
-    assert k_cache.shape[1:] == (G, k_cache.shape[2], D) and v_cache.shape[1:] == (G, k_cache.shape[2], Dv)
-    qn = torch.empty((T, H, D), dtype=torch.float32, device=qkv.device)
+    assert k_cache.shape[1:] == (G, k_cache.shape[2], D) and v_cache.shape[1:] == (G, Dv, k_cache.shape[2])
+    qn = torch.empty((T, H, D), dtype=qkv.dtype, device=qkv.device)
     N.call("vda_unit_rms_qk_cache", qn.data_ptr(), qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(),
            v_cache.data_ptr(), slot_mapping.data_ptr(), T, H, G, D, Dv, k_cache.shape[2], float(eps),
            N.dt(qkv.dtype), N.stream())
@@ -1317,21 +1317,35 @@ def sigmoid_window_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: t
                              talk: torch.Tensor, pb: torch.Tensor, scale: float, window: int, keep_first: int,
                              max_query_len: int, out_dtype: torch.dtype) -> torch.Tensor:
     """out[i, h] = sum_j sigmoid(sum_g talk[h, g] * scale * qn[i, g] . k[j, kv(g)] + pb[h]) v[j, kv(h)] over the keys
-    j <= i with i - j < window or j < keep_first (window 0: all of them).  qn fp32 [T, H, D]; talk [H, H] and pb [H]
-    fp32; returns [T, H * Dv] in ``out_dtype`` (the cache's type)."""
+    j <= i with i - j < window or j < keep_first (window 0: all of them).  qn [T, H, D] in the cache's type; talk
+    [H, H] and pb [H] fp32; returns [T, H * Dv] in ``out_dtype`` (the cache's type)."""
     if not _dev(qn):
         return R.sigmoid_window_attention(qn, k_cache, v_cache, block_table, seq_lens, query_start_loc, talk, pb,
                                           scale, window, keep_first, out_dtype)
     T, H, D = qn.shape
-    G, bs, Dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    G, Dv, bs = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     S = seq_lens.shape[0]
     assert qn.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and out_dtype == k_cache.dtype
+    assert qn.dtype == k_cache.dtype
     assert talk.dtype == torch.float32 and talk.is_contiguous() and pb.dtype == torch.float32
     out = torch.zeros((T, H * Dv), dtype=out_dtype, device=qn.device)
-    N.call("vda_sigmoid_window_attention", out.data_ptr(), qn.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-           block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(),
-           talk.data_ptr(), pb.data_ptr(), float(scale), int(window), int(keep_first), S, H, G, D, Dv, bs,
-           max(int(max_query_len), 1), N.dt(out_dtype), N.stream())
+    # 16-bit activations: q.k and weights.v on the matrix cores; fp32 (and sizes that form is not built for):
+    # plain fp32 arithmetic
+    form = envs.VDA_SIGMOID_ATTN_FORM
+    mfma = form != "plain" and bool(N.lib().vda_sigmoid_attention_mfma_ok(H, G, D, Dv, bs, N.dt(out_dtype)))
+    if form == "mfma" and not mfma:
+        raise ValueError("VDA_SIGMOID_ATTN_FORM=mfma: the matrix-core form does not take this problem")
+    args = (out.data_ptr(), qn.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+            block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(), talk.data_ptr(), pb.data_ptr(),
+            float(scale), int(window), int(keep_first), S, H, G, D, Dv, bs, max(int(max_query_len), 1),
+            N.dt(out_dtype))
+    if mfma:
+        rc = N.lib().vda_sigmoid_window_attention(*args, 1, N.stream())
+        if rc == 0:
+            return out
+        if rc > -1000 or form == "mfma":     # <= -1000: the device refused the kernel's LDS; anything else is a fault
+            raise RuntimeError(f"vda_sigmoid_window_attention (matrix-core form) failed with code {rc}")
+    N.call("vda_sigmoid_window_attention", *args, 0, N.stream())
     return out
 
 
@@ -1357,9 +1371,10 @@ def gated_delta_rule(qkv: torch.Tensor, a_raw: torch.Tensor, b_raw: torch.Tensor
     for t in (a_log, dt_bias, norm_w):
         assert t.dtype == torch.float32 and t.is_contiguous()
     out = torch.empty((T, H * Dv), dtype=qkv.dtype, device=qkv.device)
-    N.call("vda_gated_delta_rule", out.data_ptr(), out.stride(0), qkv.data_ptr(), qkv.stride(0), a_raw.data_ptr(),
-           a_raw.stride(0), b_raw.data_ptr(), b_raw.stride(0), gate_raw.data_ptr(), gate_raw.stride(0),
-           a_log.data_ptr(), dt_bias.data_ptr(), norm_w.data_ptr(), state.data_ptr(), query_start_loc.data_ptr(),
-           seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), S, H, G, D, Dv, float(eps),
-           N.dt(qkv.dtype), N.stream())
+    o_raw = torch.zeros((T, H * Dv), dtype=torch.float32, device=qkv.device)     # read-out before norm and gate
+    N.call("vda_gated_delta_rule", out.data_ptr(), out.stride(0), o_raw.data_ptr(), qkv.data_ptr(), qkv.stride(0),
+           a_raw.data_ptr(), a_raw.stride(0), b_raw.data_ptr(), b_raw.stride(0), gate_raw.data_ptr(),
+           gate_raw.stride(0), a_log.data_ptr(), dt_bias.data_ptr(), norm_w.data_ptr(), state.data_ptr(),
+           query_start_loc.data_ptr(), seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), T, S, H, G,
+           D, Dv, float(eps), N.dt(qkv.dtype), N.stream())
     return out

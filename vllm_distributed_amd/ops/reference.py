@@ -586,8 +586,8 @@ def stream_update(xs, y, mix, w_out):
 
 # ---- sigmoid attention with mixed head scores over a window plus kept first tokens ------------------
 def unit_rms_qk_and_cache(qkv, H: int, G: int, D: int, Dv: int, eps: float, k_cache, v_cache, slot_mapping):
-    """qkv [T, H*D + G*D + G*Dv] -> q / rms(q) per head as fp32 [T, H, D]; k / rms(k) and v go to the paged cache
-    (k_cache [blocks, G, bs, D], v_cache [blocks, G, bs, Dv]) at ``slot_mapping`` (negative: not stored)."""
+    """qkv [T, H*D + G*D + G*Dv] -> q / rms(q) per head as [T, H, D] (qkv's type); k / rms(k) and v go to the cache
+    (k_cache [blocks, G, bs, D], v_cache [blocks, G, Dv, bs]) at ``slot_mapping`` (negative: not stored)."""
     T = qkv.shape[0]
     q = qkv[:, : H * D].float().view(T, H, D)
     k = qkv[:, H * D: (H + G) * D].float().view(T, G, D)
@@ -599,8 +599,8 @@ def unit_rms_qk_and_cache(qkv, H: int, G: int, D: int, Dv: int, eps: float, k_ca
         ok = slot_mapping[:T] >= 0
         sl = slot_mapping[:T][ok].long()
         k_cache[sl // bs, :, sl % bs] = k[ok].to(k_cache.dtype)
-        v_cache[sl // bs, :, sl % bs] = v[ok].to(v_cache.dtype)
-    return q
+        v_cache[sl // bs, :, :, sl % bs] = v[ok].to(v_cache.dtype)
+    return q.to(qkv.dtype)
 
 
 def sigmoid_window_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, talk, pb, scale: float, window: int,
@@ -609,7 +609,7 @@ def sigmoid_window_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, t
     weight = sigmoid(mixed + pb[h]) on the visible keys (j <= i and (i - j < window or j < keep_first); window 0 =
     every earlier key), no normalisation over keys; out[i, h] = sum_j weight[h, i, j] v[j, kv(h)]."""
     T, H, D = qn.shape
-    G, bs, Dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    G, Dv, bs = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     out = torch.zeros((T, H, Dv), dtype=torch.float32, device=qn.device)
     rep = H // G
     for s in range(seq_lens.shape[0]):
@@ -621,7 +621,7 @@ def sigmoid_window_attention(qn, k_cache, v_cache, block_table, seq_lens, qsl, t
         nb = -(-sl // bs)
         blocks = block_table[s, :nb].long()
         k = k_cache[blocks].float().permute(0, 2, 1, 3).reshape(nb * bs, G, D)[:sl]
-        v = v_cache[blocks].float().permute(0, 2, 1, 3).reshape(nb * bs, G, Dv)[:sl]
+        v = v_cache[blocks].float().permute(0, 3, 1, 2).reshape(nb * bs, G, Dv)[:sl]
         kk, vv = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
         raw = torch.einsum("ihd,jhd->hij", qn[t0:t1].float(), kk) * scale
         mixed = torch.einsum("hg,gij->hij", talk.float(), raw)

@@ -54,8 +54,6 @@ class FullAttentionSpec(AttentionSpec):
     sliding_window: Optional[int] = None   # kept so hybrid models can be served with one group
     # values narrower or wider than keys (None: the key width); the V tensor then has its own size
     v_head_size: Optional[int] = None
-    # V stored [blocks, kv_heads, block, width] like K, instead of the MFMA kernels' [blocks, kv_heads, width, block]
-    token_major_v: bool = False
 
     @property
     def k_bytes_per_block(self) -> int:
@@ -69,10 +67,10 @@ class FullAttentionSpec(AttentionSpec):
 
     @property
     def type_id(self) -> str:
-        if self.v_head_size is not None or self.token_major_v:
+        if self.v_head_size is not None:
             # equal page bytes do not make equal tensors here: the split between K and V is part of the type
-            return (f"full_{self.block_size}_{self.num_kv_heads}x{self.head_size}+{self.v_head_size or self.head_size}"
-                    f"{'t' if self.token_major_v else ''}_{_dtype_size(self.dtype)}")
+            return (f"full_{self.block_size}_{self.num_kv_heads}x{self.head_size}+{self.v_head_size}"
+                    f"_{_dtype_size(self.dtype)}")
         return f"full_{self.block_size}_{self.page_size_bytes}"
 
     def max_memory_usage_bytes(self, max_model_len: int, max_num_batched_tokens: int) -> int:

@@ -566,10 +566,7 @@ class ModelRunner:
                 if vd != sp.head_size:                 # keys and values of different widths
                     half = nb * sp.k_bytes_per_block
                 k = raw[:half].view(sp.dtype).view(nb, sp.num_kv_heads, sp.block_size, sp.head_size)
-                if getattr(sp, "token_major_v", False):
-                    v = raw[half:].view(sp.dtype).view(nb, sp.num_kv_heads, sp.block_size, vd)
-                else:
-                    v = raw[half:].view(sp.dtype).view(nb, sp.num_kv_heads, vd, sp.block_size)
+                v = raw[half:].view(sp.dtype).view(nb, sp.num_kv_heads, vd, sp.block_size)
                 for n in t.shared_by:
                     self.attn_layers[n].bind_kv_cache(k, v)
                     self.kv_layer_loc[n] = (ci, off, half)
