@@ -2,8 +2,6 @@
 tests/nositar_oracle.py: every mechanism alone, then whole models through the engine's own scheduler, page pool, state
 slots and step function -- on the CPU backend (fp32) and, marked gpu, through the HIP kernels (fp32 and bf16).
 Small random models are written to disk as checkpoints, so the loader and the configuration reader run too."""
-import math
-
 import pytest
 import torch
 
@@ -112,7 +110,6 @@ def test_sigmoid_attention_paged(dev, H, G, D, E, window, keep):
     whole prompt -- against the dense oracle of each sequence."""
     bs, eps, scale = 4, 1e-5, 0.3
     lens, news = [23, 37, 14], [1, 9, 14]
-    width = (H + 2 * G) * D if D == E else None
     C = H * D + G * D + G * E
     seqs = [torch.randn(n, C) for n in lens]
     talk, pb = torch.eye(H) + 0.4 * torch.randn(H, H), torch.randn(H) - 1.0

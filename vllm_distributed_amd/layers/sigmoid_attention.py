@@ -72,7 +72,8 @@ class SigmoidWindowAttention(nn.Module):
                                        md.slot_mapping[:n])
         out = ops.sigmoid_window_attention(qn, self.k_cache, self.v_cache, md.block_table[:S], md.seq_lens[:S],
                                            md.query_start_loc[:S + 1], self.talk, self.score_bias, self.scale,
-                                           self.window, self.keep_first, md.max_query_len, qkv.dtype)
+                                           self.window, self.keep_first, md.max_query_len, qkv.dtype,
+                                           max_seq_len=md.max_seq_len)
         if n < T:
             out = torch.cat([out, out.new_zeros((T - n, out.shape[1]))], dim=0)
         return self.o_proj(out)

@@ -1315,7 +1315,7 @@ def unit_rms_qk_and_cache(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, ep
 def sigmoid_window_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                              block_table: torch.Tensor, seq_lens: torch.Tensor, query_start_loc: torch.Tensor,
                              talk: torch.Tensor, pb: torch.Tensor, scale: float, window: int, keep_first: int,
-                             max_query_len: int, out_dtype: torch.dtype) -> torch.Tensor:
+                             max_query_len: int, out_dtype: torch.dtype, max_seq_len: int = 0) -> torch.Tensor:
     """out[i, h] = sum_j sigmoid(sum_g talk[h, g] * scale * qn[i, g] . k[j, kv(g)] + pb[h]) v[j, kv(h)] over the keys
     j <= i with i - j < window or j < keep_first (window 0: all of them).  qn [T, H, D] in the cache's type; talk
     [H, H] and pb [H] fp32; returns [T, H * Dv] in ``out_dtype`` (the cache's type)."""
@@ -1340,12 +1340,21 @@ def sigmoid_window_attention(qn: torch.Tensor, k_cache: torch.Tensor, v_cache: t
             float(scale), int(window), int(keep_first), S, H, G, D, Dv, bs, max(int(max_query_len), 1),
             N.dt(out_dtype))
     if mfma:
-        rc = N.lib().vda_sigmoid_window_attention(*args, 1, N.stream())
+        # few query tiles (decoding): deal the 128-key steps to several workgroups per tile; their partial sums add
+        tiles = -(-max(int(max_query_len), 1) // 16) * S
+        parts, part = 1, None
+        if tiles < 128:
+            keys = (window + 15 if window > 0 else max(int(max_seq_len), 1))
+            steps = -(-keys // 128) + 1 + (1 if window > 0 and keep_first > 0 else 0)
+            parts = max(1, min(steps, 16, 256 // tiles))
+            if parts > 1:
+                part = torch.zeros((parts, T * H * Dv), dtype=torch.float32, device=qn.device)
+        rc = N.lib().vda_sigmoid_window_attention(*args, 1, N.ptr(part), T * H * Dv, parts, N.stream())
         if rc == 0:
             return out
         if rc > -1000 or form == "mfma":     # <= -1000: the device refused the kernel's LDS; anything else is a fault
             raise RuntimeError(f"vda_sigmoid_window_attention (matrix-core form) failed with code {rc}")
-    N.call("vda_sigmoid_window_attention", *args, 0, N.stream())
+    N.call("vda_sigmoid_window_attention", *args, 0, None, 0, 1, N.stream())
     return out
 
 
@@ -1372,7 +1381,10 @@ def gated_delta_rule(qkv: torch.Tensor, a_raw: torch.Tensor, b_raw: torch.Tensor
         assert t.dtype == torch.float32 and t.is_contiguous()
     out = torch.empty((T, H * Dv), dtype=qkv.dtype, device=qkv.device)
     o_raw = torch.zeros((T, H * Dv), dtype=torch.float32, device=qkv.device)     # read-out before norm and gate
-    N.call("vda_gated_delta_rule", out.data_ptr(), out.stride(0), o_raw.data_ptr(), qkv.data_ptr(), qkv.stride(0),
+    Dp = N.lib().vda_delta_rule_padded_dim(D)
+    prep = torch.empty(T * ((2 * G + H) * Dp + 2 * H), dtype=torch.float32, device=qkv.device)
+    N.call("vda_gated_delta_rule", out.data_ptr(), out.stride(0), o_raw.data_ptr(), prep.data_ptr(), qkv.data_ptr(),
+           qkv.stride(0),
            a_raw.data_ptr(), a_raw.stride(0), b_raw.data_ptr(), b_raw.stride(0), gate_raw.data_ptr(),
            gate_raw.stride(0), a_log.data_ptr(), dt_bias.data_ptr(), norm_w.data_ptr(), state.data_ptr(),
            query_start_loc.data_ptr(), seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), T, S, H, G,

@@ -6,92 +6,51 @@
 // beta = sigmoid(b).  The read-out sees the token's own write.  The output is RMS-normalised over Dv, scaled by a
 // weight shared by the heads and gated by sigmoid(gate).
 //
-// Every column of S evolves on its own given (q, k, decay, beta), so a workgroup owns one (sequence, head, group of
-// 32 columns) and its threads own columns: four adjacent lanes share a column, NR = D/4 rows each in registers, and
-// the two dot products of a step (k . dS and q . dS, taken on the decayed state before the write, o = q . dS +
-// (q . k) u) are summed over the four lanes together.  Tokens are walked in chunks of 16: the chunk's unit vectors,
-// decays and gates are computed once by all threads (fp32) into LDS -- all loads of a chunk issued together, rows
-// padded so that the four lanes of a column read different banks with 16-byte loads -- then every thread runs its
-// column through the chunk.  The read-out goes
-// to an fp32 scratch; a second small kernel normalises it over the head's columns and gates it.
+// Two kernels and a small epilogue:
+//   prepare  (parallel over tokens)  unit vectors q^, k^ per q/k head, decays per head and key channel, beta and
+//            q^ . k^ per head, all fp32, rows padded with zeros to a multiple of 16 channels;
+//   scan     every column of S evolves on its own given (q^, k^, decay, beta), so a workgroup owns one (sequence,
+//            head, 16 columns) and sixteen adjacent lanes share a column, NR = D/16 rows each in registers.  The two
+//            dot products of a step (k^ . dS and q^ . dS on the decayed state, o = q^ . dS + (q^ . k^) u) are summed
+//            over the sixteen lanes with DPP row operations.  The prepared vectors of 32 tokens sit in LDS while
+//            the next 32 are on their way from memory, so a step is one short dependent chain of register work.
+//   epilogue normalises the read-out over the head's columns, applies the weight and the gate.
 // The batch description is the one of the other recurrent kernels (qsl, seq_lens, slot in column 0 of the table;
 // a sequence carries state in when seq_len - new_tokens > 0), so prompts, portions of prompts, single decoded
 // tokens and mixtures of them are one code path, and the state after a token does not depend on how the
 // sequence was cut.
 #include "common.h"
 
-#define DR_CT 16
-
 __device__ __forceinline__ float dr_softplus(float v) { return v > 20.f ? v : log1pf(expf(v)); }
 __device__ __forceinline__ float dr_sigmoid(float v) { return 1.f / (1.f + expf(-v)); }
 
-// LDS row of one token's vector: the four row groups (one per lane of a column) sit NR + pad floats apart so that
-// their 16-byte reads fall into different banks
-template <int NR> struct DrRow {
-  static constexpr int PS = NR + (NR == 12 ? 8 : 4);
-  static constexpr int LEN = 4 * PS;
-};
+// sum over the 16 lanes of a DPP row, result in every lane
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+  return v;
+}
 
-// grid (heads, sequences, column groups); block 4 * Cw threads, Cw columns of S per workgroup.  Writes the raw
-// read-out o (fp32) to `o_raw` [T, H * Dv]; vda_gated_delta_rule's second kernel normalises and gates it.
-template <typename T, int NR>
-__global__ __launch_bounds__(256) void gated_delta_rule_kernel(
-    float* __restrict__ o_raw, const T* __restrict__ qkv, long qkv_stride, const T* __restrict__ a_raw,
-    long a_stride, const T* __restrict__ b_raw, long b_stride, const float* __restrict__ a_log,
-    const float* __restrict__ dt_bias, float* __restrict__ state, const int* __restrict__ qsl,
-    const int* __restrict__ seq_lens, const int* __restrict__ slot_table, long st_stride, int H, int G, int D,
-    int Dv, int Cw) {
-  constexpr int PS = DrRow<NR>::PS, RL = DrRow<NR>::LEN;
-  extern __shared__ __align__(16) float lds[];
-  const int nthreads = blockDim.x;
-  float* qh = lds;                      // [CT][RL]
-  float* kh = qh + DR_CT * RL;          // [CT][RL]
-  float* gh = kh + DR_CT * RL;          // [CT][RL]
-  float* vv = gh + DR_CT * RL;          // [CT][Cw]
-  float* qk = vv + DR_CT * Cw;          // [CT]
-  float* bt = qk + DR_CT;               // [CT]
-
-  const int h = blockIdx.x, s = blockIdx.y, col0 = blockIdx.z * Cw, tid = threadIdx.x;
-  const int sl = seq_lens[s];
-  if (sl <= 0) return;
-  const int t0 = qsl[s], L = qsl[s + 1] - t0;
-  if (L <= 0) return;
-  const int c = h / (H / G);            // q / k head of this head
-  const int col = col0 + (tid >> 2), part = tid & 3;
-  const int lane = tid & 63, wave = tid >> 6, nw = nthreads >> 6;
-  const bool has_col = col < Dv;
-  float* Scol = state + (((long)slot_table[s * st_stride] * H + h) * Dv + (has_col ? col : 0)) * D + part * NR;
-  float S[NR];
-  const bool carry = sl - L > 0;
-#pragma unroll
-  for (int i = 0; i < NR; ++i) S[i] = (carry && has_col && part * NR + i < D) ? Scol[i] : 0.f;
-  const float a_scale = expf(a_log[h]);
+// grid: tokens; one wave per (token, vector): G query vectors, G key vectors (with their dot products), H decays
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_kernel(
+    float* __restrict__ qhat, float* __restrict__ khat, float* __restrict__ dec, float* __restrict__ sc,
+    const T* __restrict__ qkv, long qkv_stride, const T* __restrict__ a_raw, long a_stride,
+    const T* __restrict__ b_raw, long b_stride, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    int H, int G, int D, int Dp) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float q_scale = 1.f / sqrtf((float)D);
-
-  for (int cs = 0; cs < L; cs += DR_CT) {
-    const int nt = min(DR_CT, L - cs);
-    // ---- the chunk's inputs: every thread loads its share at once (one trip to memory per chunk) ------------
-    for (int e = tid; e < nt * D; e += nthreads) {
-      const int tt = e / D, d = e - tt * D;
-      const long t = t0 + cs + tt;
-      const int at = tt * RL + (d / NR) * PS + d % NR;
-      qh[at] = (float)qkv[t * qkv_stride + (long)c * D + d];
-      kh[at] = (float)qkv[t * qkv_stride + (long)(G + c) * D + d];
-      gh[at] = (float)a_raw[t * a_stride + (long)h * D + d];
-    }
-    for (int e = tid; e < nt * Cw; e += nthreads) {
-      const int tt = e / Cw, j = e - tt * Cw;
-      vv[e] = col0 + j < Dv ? (float)qkv[(long)(t0 + cs + tt) * qkv_stride + (long)2 * G * D + (long)h * Dv + col0 + j]
-                            : 0.f;
-    }
-    if (tid < nt) bt[tid] = dr_sigmoid((float)b_raw[(long)(t0 + cs + tid) * b_stride + h]);
-    __syncthreads();
-    // ---- unit vectors and decays in place, one wave per token ---------------------------------------------------
-    for (int tt = wave; tt < nt; tt += nw) {
+  const int rep = H / G;
+  for (int v = wave; v < G + H; v += 4) {
+    if (v < G) {
+      const T* qr = qkv + t * qkv_stride + (long)v * D;
+      const T* kr = qkv + t * qkv_stride + (long)(G + v) * D;
       float sq = 0.f, sk = 0.f;
       for (int d = lane; d < D; d += 64) {
-        const int at = tt * RL + (d / NR) * PS + d % NR;
-        const float a = qh[at], b = kh[at];
+        const float a = (float)qr[d], b = (float)kr[d];
         sq += a * a;
         sk += b * b;
       }
@@ -99,61 +58,139 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
       sk = wave_sum(sk);
       const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.f / sqrtf(sk + 1e-6f);
       float dot = 0.f;
-      for (int d = lane; d < 4 * NR; d += 64) {
-        const int at = tt * RL + (d / NR) * PS + d % NR;
-        float a = 0.f, b = 0.f, g = 0.f;
-        if (d < D) {
-          a = qh[at] * rq;
-          b = kh[at] * rk;
-          g = expf(-a_scale * dr_softplus(gh[at] + dt_bias[(long)h * D + d]));
-        }
-        qh[at] = a;
-        kh[at] = b;
-        gh[at] = g;
+      for (int d = lane; d < Dp; d += 64) {
+        const float a = d < D ? (float)qr[d] * rq : 0.f, b = d < D ? (float)kr[d] * rk : 0.f;
+        qhat[(t * G + v) * Dp + d] = a;
+        khat[(t * G + v) * Dp + d] = b;
         dot += a * b;
       }
       dot = wave_sum(dot);
-      if (lane == 0) qk[tt] = dot;
+      // per head: [beta, q^ . k^]
+      for (int h = v * rep + lane; h < (v + 1) * rep; h += 64) {
+        sc[(t * H + h) * 2] = dr_sigmoid((float)b_raw[t * b_stride + h]);
+        sc[(t * H + h) * 2 + 1] = dot;
+      }
+    } else {
+      const int h = v - G;
+      const float a_scale = expf(a_log[h]);
+      for (int d = lane; d < Dp; d += 64)
+        dec[(t * H + h) * Dp + d] =
+            d < D ? expf(-a_scale * dr_softplus((float)a_raw[t * a_stride + (long)h * D + d] + dt_bias[(long)h * D + d]))
+                  : 0.f;
     }
+  }
+}
+
+
+// grid (heads, sequences, groups of 16 columns); block 256 = 16 columns x 16 lanes.  The prepared vectors of 32
+// tokens are staged in LDS; the next 32 are on their way from memory (into registers) while these are computed.
+template <typename T, int NR>
+__global__ __launch_bounds__(256) void gated_delta_rule_kernel(
+    float* __restrict__ o_raw, const T* __restrict__ qkv, long qkv_stride, const float* __restrict__ qhat,
+    const float* __restrict__ khat, const float* __restrict__ dec, const float* __restrict__ sc,
+    float* __restrict__ state, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
+    const int* __restrict__ slot_table, long st_stride, int H, int G, int D, int Dv) {
+  constexpr int Dp = 16 * NR;
+  constexpr int DR_CT = NR >= 16 ? 16 : 32;            // tokens staged in LDS at a time (48 KiB at most)
+  constexpr int NV = DR_CT * 16 / 256;                 // value elements a thread carries per chunk
+  constexpr int VPT = DR_CT * Dp / 4;                  // float4 per staged vector kind
+  constexpr int PF = (3 * VPT + 255) / 256;            // float4 a thread carries per chunk
+  __shared__ __align__(16) float kqg[3 * DR_CT * Dp];  // k^ | q^ | decay, [kind][token][Dp]
+  __shared__ float vv[DR_CT * 16];
+  __shared__ float sc2[DR_CT * 2];
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+  const int sl = seq_lens[s];
+  if (sl <= 0) return;
+  const int t0 = qsl[s], L = qsl[s + 1] - t0;
+  if (L <= 0) return;
+  const int c = h / (H / G);
+  const int col0 = blockIdx.z * 16;
+  const int col = col0 + (tid >> 4), part = tid & 15;
+  const bool has_col = col < Dv;
+  float* Scol = state + (((long)slot_table[s * st_stride] * H + h) * Dv + (has_col ? col : Dv - 1)) * D + part * NR;
+  float S[NR];
+  const bool carry = sl - L > 0;
+#pragma unroll
+  for (int i = 0; i < NR; ++i) S[i] = (carry && part * NR + i < D) ? Scol[i] : 0.f;
+
+  f32x4 pre[PF];
+  float pv[NV], ps = 0.f;
+  auto prefetch = [&](int cs) {
+    const int nt = min(DR_CT, L - cs);
+#pragma unroll
+    for (int n = 0; n < PF; ++n) {
+      const int e = tid + n * 256;
+      f32x4 x = {0.f, 0.f, 0.f, 0.f};
+      if (e < 3 * VPT) {
+        const int kind = e / VPT, rem = e - kind * VPT, tt = rem / (Dp / 4), j = rem - tt * (Dp / 4);
+        if (tt < nt) {
+          const long t = t0 + cs + tt;
+          const float* src = kind == 0 ? khat + (t * G + c) * Dp : kind == 1 ? qhat + (t * G + c) * Dp
+                                                                             : dec + (t * H + h) * Dp;
+          x = *reinterpret_cast<const f32x4*>(src + 4 * j);
+        }
+      }
+      pre[n] = x;
+    }
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int e = tid + n * 256, tt = e >> 4, j = e & 15;
+      pv[n] = (tt < nt && col0 + j < Dv)
+                  ? (float)qkv[(long)(t0 + cs + tt) * qkv_stride + (long)2 * G * D + (long)h * Dv + col0 + j] : 0.f;
+    }
+    if (tid < 2 * DR_CT) ps = (tid >> 1) < nt ? sc[((long)(t0 + cs + (tid >> 1)) * H + h) * 2 + (tid & 1)] : 0.f;
+  };
+
+  prefetch(0);
+  for (int cs = 0; cs < L; cs += DR_CT) {
+    const int nt = min(DR_CT, L - cs);
+    __syncthreads();                                   // the previous chunk has been read by everybody
+#pragma unroll
+    for (int n = 0; n < PF; ++n) {
+      const int e = tid + n * 256;
+      if (e < 3 * VPT) *reinterpret_cast<f32x4*>(kqg + 4 * e) = pre[n];
+    }
+#pragma unroll
+    for (int n = 0; n < NV; ++n) vv[tid + n * 256] = pv[n];
+    if (tid < 2 * DR_CT) sc2[tid] = ps;
     __syncthreads();
-    // ---- the recurrence: every thread its rows of one column ------------------------------------------------
+    if (cs + DR_CT < L) prefetch(cs + DR_CT);
     for (int tt = 0; tt < nt; ++tt) {
-      const f32x4* kp = reinterpret_cast<const f32x4*>(kh + tt * RL + part * PS);
-      const f32x4* qp = reinterpret_cast<const f32x4*>(qh + tt * RL + part * PS);
-      const f32x4* gp = reinterpret_cast<const f32x4*>(gh + tt * RL + part * PS);
-      f32x4 kreg[NR / 4];
-      float r0 = 0.f, r1 = 0.f, p0 = 0.f, p1 = 0.f;
+      const float* kp = kqg + tt * Dp + part * NR;
+      const float* qp = kp + DR_CT * Dp;
+      const float* gp = qp + DR_CT * Dp;
+      float kr[NR], r = 0.f, p = 0.f;
+      if constexpr (NR >= 4) {
 #pragma unroll
-      for (int i = 0; i < NR / 4; ++i) {
-        const f32x4 g4 = gp[i], k4 = kp[i], q4 = qp[i];
-        kreg[i] = k4;
-        const float s0 = S[4 * i] * g4[0], s1 = S[4 * i + 1] * g4[1], s2 = S[4 * i + 2] * g4[2],
-                    s3 = S[4 * i + 3] * g4[3];
-        S[4 * i] = s0;
-        S[4 * i + 1] = s1;
-        S[4 * i + 2] = s2;
-        S[4 * i + 3] = s3;
-        r0 += s0 * k4[0] + s2 * k4[2];
-        r1 += s1 * k4[1] + s3 * k4[3];
-        p0 += s0 * q4[0] + s2 * q4[2];
-        p1 += s1 * q4[1] + s3 * q4[3];
-      }
-      float r = r0 + r1, p = p0 + p1;
-      r += __shfl_xor(r, 1, 64);
-      p += __shfl_xor(p, 1, 64);
-      r += __shfl_xor(r, 2, 64);
-      p += __shfl_xor(p, 2, 64);
-      const float u = bt[tt] * (vv[tt * Cw + (tid >> 2)] - r);
+        for (int i = 0; i < NR / 4; ++i) {
+          const f32x4 k4 = reinterpret_cast<const f32x4*>(kp)[i], q4 = reinterpret_cast<const f32x4*>(qp)[i],
+                      g4 = reinterpret_cast<const f32x4*>(gp)[i];
 #pragma unroll
-      for (int i = 0; i < NR / 4; ++i) {
-        S[4 * i] += kreg[i][0] * u;
-        S[4 * i + 1] += kreg[i][1] * u;
-        S[4 * i + 2] += kreg[i][2] * u;
-        S[4 * i + 3] += kreg[i][3] * u;
+          for (int j = 0; j < 4; ++j) {
+            const float sd = S[4 * i + j] * g4[j];
+            S[4 * i + j] = sd;
+            kr[4 * i + j] = k4[j];
+            r += sd * k4[j];
+            p += sd * q4[j];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          const float sd = S[i] * gp[i];
+          S[i] = sd;
+          kr[i] = kp[i];
+          r += sd * kp[i];
+          p += sd * qp[i];
+        }
       }
-      if (part == 0 && has_col) o_raw[(long)(t0 + cs + tt) * H * Dv + (long)h * Dv + col] = p + qk[tt] * u;
+      r = row16_sum(r);
+      p = row16_sum(p);
+      const float u = sc2[2 * tt] * (vv[tt * 16 + (tid >> 4)] - r);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) S[i] += kr[i] * u;
+      if (part == 0 && has_col) o_raw[(long)(t0 + cs + tt) * H * Dv + (long)h * Dv + col] = p + sc2[2 * tt + 1] * u;
     }
-    __syncthreads();
   }
   if (has_col) {
 #pragma unroll
@@ -186,67 +223,66 @@ __global__ __launch_bounds__(256) void delta_out_norm_gate_kernel(T* __restrict_
 }
 
 template <typename T>
-static int launch_delta_rule(int NRsel, dim3 grid, dim3 block, hipStream_t st, float* o_raw, const void* qkv,
-                             long qkv_stride, const void* a_raw, long a_stride, const void* b_raw, long b_stride,
-                             const float* a_log, const float* dt_bias, float* state, const int* qsl,
-                             const int* seq_lens, const int* slot_table, long st_stride, int H, int G, int D, int Dv,
-                             int Cw) {
-#define L(NRV)                                                                                                        \
-  do {                                                                                                                \
-    const size_t lds = ((size_t)DR_CT * (3 * DrRow<NRV>::LEN + Cw) + 2 * DR_CT) * sizeof(float);                      \
-    if (lds > 48 * 1024) {                                                                                            \
-      hipError_t e = hipFuncSetAttribute((const void*)gated_delta_rule_kernel<T, NRV>,                               \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                       \
-      if (e != hipSuccess) return (int)e;                                                                             \
-    }                                                                                                                 \
-    hipLaunchKernelGGL((gated_delta_rule_kernel<T, NRV>), grid, block, lds, st, o_raw, (const T*)qkv, qkv_stride,     \
-                       (const T*)a_raw, a_stride, (const T*)b_raw, b_stride, a_log, dt_bias, state, qsl, seq_lens,    \
-                       slot_table, st_stride, H, G, D, Dv, Cw);                                                       \
-  } while (0)
-  switch (NRsel) {
+static int launch_delta_rule(int NR, dim3 grid, hipStream_t st, float* o_raw, const void* qkv, long qkv_stride,
+                             const float* qhat, const float* khat, const float* dec, const float* sc, float* state,
+                             const int* qsl, const int* seq_lens, const int* slot_table, long st_stride, int H, int G,
+                             int D, int Dv) {
+#define L(NRV)                                                                                                     \
+  hipLaunchKernelGGL((gated_delta_rule_kernel<T, NRV>), grid, dim3(256), 0, st, o_raw, (const T*)qkv, qkv_stride,  \
+                     qhat, khat, dec, sc, state, qsl, seq_lens, slot_table, st_stride, H, G, D, Dv)
+  switch (NR) {
+    case 1: L(1); break;
+    case 2: L(2); break;
     case 4: L(4); break;
     case 8: L(8); break;
-    case 12: L(12); break;
     case 16: L(16); break;
-    case 24: L(24); break;
-    case 32: L(32); break;
-    case 48: L(48); break;
-    case 64: L(64); break;
     default: return -2;
   }
 #undef L
   return 0;
 }
 
-// o_raw: fp32 scratch [T, H * Dv] of the caller
-VDA_EXPORT int vda_gated_delta_rule(void* out, long o_stride, float* o_raw, const void* qkv, long qkv_stride,
-                                    const void* a_raw, long a_stride, const void* b_raw, long b_stride,
-                                    const void* gate_raw, long g_stride, const float* a_log, const float* dt_bias,
-                                    const float* norm_w, float* state, const int* qsl, const int* seq_lens,
-                                    const int* slot_table, long st_stride, int T_tokens, int S, int H, int G, int D,
-                                    int Dv, float eps, int dtype, hipStream_t st) {
+// channels per lane of the scan for key width D (D <= 256), and the padded row length of the prepared vectors
+VDA_EXPORT int vda_delta_rule_padded_dim(int D) {
+  int NR = 1;
+  while (16 * NR < D) NR *= 2;
+  return 16 * NR;
+}
+
+// o_raw: fp32 [T, H * Dv]; prep: fp32 scratch of T * ((2 G + H) * Dp + 2 H) floats, Dp = vda_delta_rule_padded_dim(D)
+VDA_EXPORT int vda_gated_delta_rule(void* out, long o_stride, float* o_raw, float* prep, const void* qkv,
+                                    long qkv_stride, const void* a_raw, long a_stride, const void* b_raw,
+                                    long b_stride, const void* gate_raw, long g_stride, const float* a_log,
+                                    const float* dt_bias, const float* norm_w, float* state, const int* qsl,
+                                    const int* seq_lens, const int* slot_table, long st_stride, int T_tokens, int S,
+                                    int H, int G, int D, int Dv, float eps, int dtype, hipStream_t st) {
   if (S <= 0 || T_tokens <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D < 1 || D > 256 || Dv < 1) return -1;
-  static const int sizes[] = {4, 8, 12, 16, 24, 32, 48, 64};
-  int NR = 0;
-  for (int v : sizes)
-    if (4 * v >= D) { NR = v; break; }
-  // columns per workgroup: 32 (two waves) unless the head is narrower; wide rows keep 16 to stay within registers
-  int Cw = NR > 32 ? 16 : 32;
-  if (Dv <= 16) Cw = 16;
-  dim3 grid(H, S, (Dv + Cw - 1) / Cw), block(4 * Cw);
+  const int Dp = vda_delta_rule_padded_dim(D), NR = Dp / 16;
+  float* qhat = prep;
+  float* khat = qhat + (size_t)T_tokens * G * Dp;
+  float* dec = khat + (size_t)T_tokens * G * Dp;
+  float* sc = dec + (size_t)T_tokens * H * Dp;
+#define LP(TT) hipLaunchKernelGGL((delta_prepare_kernel<TT>), dim3(T_tokens), dim3(256), 0, st, qhat, khat, dec, sc, \
+                                  (const TT*)qkv, qkv_stride, (const TT*)a_raw, a_stride, (const TT*)b_raw, b_stride, \
+                                  a_log, dt_bias, H, G, D, Dp)
+  if (dtype == VDA_BF16) LP(bf16_t);
+  else if (dtype == VDA_F16) LP(f16_t);
+  else if (dtype == VDA_F32) LP(float);
+  else return -3;
+#undef LP
+  VDA_CHECK_LAUNCH();
+  dim3 grid(H, S, (Dv + 15) / 16);
   int rc;
   if (dtype == VDA_BF16)
-    rc = launch_delta_rule<bf16_t>(NR, grid, block, st, o_raw, qkv, qkv_stride, a_raw, a_stride, b_raw, b_stride,
-                                   a_log, dt_bias, state, qsl, seq_lens, slot_table, st_stride, H, G, D, Dv, Cw);
+    rc = launch_delta_rule<bf16_t>(NR, grid, st, o_raw, qkv, qkv_stride, qhat, khat, dec, sc, state, qsl, seq_lens,
+                                   slot_table, st_stride, H, G, D, Dv);
   else if (dtype == VDA_F16)
-    rc = launch_delta_rule<f16_t>(NR, grid, block, st, o_raw, qkv, qkv_stride, a_raw, a_stride, b_raw, b_stride,
-                                  a_log, dt_bias, state, qsl, seq_lens, slot_table, st_stride, H, G, D, Dv, Cw);
-  else if (dtype == VDA_F32)
-    rc = launch_delta_rule<float>(NR, grid, block, st, o_raw, qkv, qkv_stride, a_raw, a_stride, b_raw, b_stride,
-                                  a_log, dt_bias, state, qsl, seq_lens, slot_table, st_stride, H, G, D, Dv, Cw);
+    rc = launch_delta_rule<f16_t>(NR, grid, st, o_raw, qkv, qkv_stride, qhat, khat, dec, sc, state, qsl, seq_lens,
+                                  slot_table, st_stride, H, G, D, Dv);
   else
-    return -3;
+    rc = launch_delta_rule<float>(NR, grid, st, o_raw, qkv, qkv_stride, qhat, khat, dec, sc, state, qsl, seq_lens,
+                                  slot_table, st_stride, H, G, D, Dv);
   if (rc) return rc;
   VDA_CHECK_LAUNCH();
   const long rows = (long)T_tokens * H;

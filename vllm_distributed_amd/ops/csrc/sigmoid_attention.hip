@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
     T* __restrict__ out, const T* __restrict__ qn, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_table, long bt_stride, const int* __restrict__ seq_lens,
     const int* __restrict__ qsl, const float* __restrict__ talk, const float* __restrict__ pb, float scale,
-    int window, int keep_first, int H, int G, int D, int Dv, int bs) {
+    int window, int keep_first, int H, int G, int D, int Dv, int bs, float* __restrict__ part, long part_stride) {
   using V8 = typename Vec<T>::v8;
   constexpr int HPW = MAXH / 4;                 // heads a wave accumulates
   extern __shared__ __align__(16) unsigned char smem[];
@@ -236,7 +236,9 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
   const int n_keep = (ka + 127) / 128, n_win = (p1 - lo_al + 127) / 128;
   const int krow0 = 8 * (r >> 2) + (r & 3);
   const int pi = p0 + r;                        // position of this lane's query column
-  for (int step = 0; step < n_keep + n_win; ++step) {
+  // few query tiles (decoding): the key steps are dealt to gridDim.z workgroups, whose partial sums -- nothing is
+  // normalised over keys, so they simply add -- go to `part` and are summed in a fixed order afterwards
+  for (int step = blockIdx.z; step < n_keep + n_win; step += gridDim.z) {
     const bool keep = step < n_keep;
     const int kb = keep ? step * 128 : lo_al + (step - n_keep) * 128;
     const int jlo = keep ? 0 : lo, jhi = keep ? ka : p1;        // keys of this range that count
@@ -355,13 +357,16 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
     for (int a = 0; a < HPW; ++a) {
       const int h = wave * HPW + a;
       if (h < H) {
-        T* op = out + (long)(t0 + i0 + r) * H * Dv + (long)h * Dv;
+        const long at = (long)(t0 + i0 + r) * H * Dv + (long)h * Dv;
 #pragma unroll
         for (int n = 0; n < NT; ++n)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const int d = n * 16 + 4 * g4 + j;
-            if (d < Dv) op[d] = (T)acc[a][n][j];
+            if (d < Dv) {
+              if (part) part[blockIdx.z * part_stride + at + d] = acc[a][n][j];
+              else out[at + d] = (T)acc[a][n][j];
+            }
           }
       }
     }
@@ -369,10 +374,20 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
 }
 
 template <typename T>
+__global__ __launch_bounds__(256) void sum_parts_kernel(T* __restrict__ out, const float* __restrict__ part,
+                                                        long n, long part_stride, int parts) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float a = 0.f;
+  for (int z = 0; z < parts; ++z) a += part[z * part_stride + i];
+  out[i] = (T)a;
+}
+
+template <typename T>
 static int launch_sigmoid_mfma(dim3 grid, hipStream_t st, void* out, const void* qn, const void* k_cache,
                                const void* v_cache, const int* block_table, long bt_stride, const int* seq_lens,
                                const int* qsl, const float* talk, const float* pb, float scale, int window,
-                               int keep_first, int H, int G, int D, int Dv, int bs) {
+                               int keep_first, int H, int G, int D, int Dv, int bs, float* part, long part_stride) {
   const int MAXH = H <= 8 ? 8 : 16, KS = D <= 64 ? 2 : 4, NT = Dv <= 64 ? 4 : 8;
   const size_t lds = (size_t)MAXH * 4 * 64 * 16;
 #define LM(MH, KK, NN)                                                                                              \
@@ -385,7 +400,7 @@ static int launch_sigmoid_mfma(dim3 grid, hipStream_t st, void* out, const void*
     hipLaunchKernelGGL((sigmoid_attention_mfma_kernel<T, MH, KK, NN>), grid, dim3(256), lds, st, (T*)out,           \
                        (const T*)qn,                                                                                \
                        (const T*)k_cache, (const T*)v_cache, block_table, bt_stride, seq_lens, qsl, talk, pb,       \
-                       scale, window, keep_first, H, G, D, Dv, bs);                                                 \
+                       scale, window, keep_first, H, G, D, Dv, bs, part, part_stride);                              \
   } while (0)
 #define LK(MH, KK) do { if (NT == 4) LM(MH, KK, 4); else LM(MH, KK, 8); } while (0)
 #define LH(MH) do { if (KS == 2) LK(MH, 2); else LK(MH, 4); } while (0)
@@ -393,6 +408,12 @@ static int launch_sigmoid_mfma(dim3 grid, hipStream_t st, void* out, const void*
 #undef LH
 #undef LK
 #undef LM
+  if (part) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL((sum_parts_kernel<T>), dim3((unsigned)((part_stride + 255) / 256)), dim3(256), 0, st, (T*)out,
+                       part, part_stride, part_stride, (int)grid.z);
+  }
   return 0;
 }
 
@@ -406,17 +427,22 @@ VDA_EXPORT int vda_sigmoid_window_attention(void* out, const void* qn, const voi
                                             const int* block_table, long bt_stride, const int* seq_lens,
                                             const int* qsl, const float* talk, const float* pb, float scale,
                                             int window, int keep_first, int S, int H, int G, int D, int Dv, int bs,
-                                            int max_q, int dtype, int form, hipStream_t st) {
+                                            int max_q, int dtype, int form, float* part, long part_stride,
+                                            int parts, hipStream_t st) {
   if (S <= 0 || max_q <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G) return -1;
   if (form == 1) {              // MFMA form
     if (!vda_sigmoid_attention_mfma_ok(H, G, D, Dv, bs, dtype)) return -2;
-    dim3 grid((max_q + 15) / 16, S);
+    // parts > 1: `part` holds parts x part_stride zeroed floats (part_stride = tokens * H * Dv)
+    dim3 grid((max_q + 15) / 16, S, part && parts > 1 ? parts : 1);
+    float* pp = grid.z > 1 ? part : nullptr;
     int rc = dtype == VDA_BF16
                  ? launch_sigmoid_mfma<bf16_t>(grid, st, out, qn, k_cache, v_cache, block_table, bt_stride, seq_lens,
-                                               qsl, talk, pb, scale, window, keep_first, H, G, D, Dv, bs)
+                                               qsl, talk, pb, scale, window, keep_first, H, G, D, Dv, bs, pp,
+                                               part_stride)
                  : launch_sigmoid_mfma<f16_t>(grid, st, out, qn, k_cache, v_cache, block_table, bt_stride, seq_lens,
-                                              qsl, talk, pb, scale, window, keep_first, H, G, D, Dv, bs);
+                                              qsl, talk, pb, scale, window, keep_first, H, G, D, Dv, bs, pp,
+                                              part_stride);
     if (rc) return rc;
     VDA_CHECK_LAUNCH();
     return 0;

@@ -87,9 +87,10 @@ _SIGS = {
     "vda_stream_embed": [P, P, P, F, I, I, I, L, I, P],
     "vda_stream_step": [P, P, L, P, P, P, P, P, F, I, I, I, L, I, I, P],
     "vda_unit_rms_qk_cache": [P, P, L, P, P, P, I, I, I, I, I, I, F, I, P],
-    "vda_sigmoid_window_attention": [P, P, P, P, P, L, P, P, P, P, F, I, I, I, I, I, I, I, I, I, I, I, P],
+    "vda_sigmoid_window_attention": [P, P, P, P, P, L, P, P, P, P, F, I, I, I, I, I, I, I, I, I, I, I, P, L, I, P],
     "vda_sigmoid_attention_mfma_ok": [I, I, I, I, I, I],
-    "vda_gated_delta_rule": [P, L, P, P, L, P, L, P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, I, P],
+    "vda_gated_delta_rule": [P, L, P, P, P, L, P, L, P, L, P, L, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, I, P],
+    "vda_delta_rule_padded_dim": [I],
     "vda_selective_scan": [P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, L, L, L, L, L, L, I, I, I, I, I, I, P, P,
                            I, P],
 }
