@@ -103,7 +103,7 @@ def test_streams_read_write(dev, n):
 
 
 @pytest.mark.parametrize("dev", DEVICES)
-@pytest.mark.parametrize("H,G,D,E,window,keep", [(4, 2, 16, 16, 9, 2), (3, 3, 20, 8, 5, 0), (8, 2, 48, 40, 40, 6),
+@pytest.mark.parametrize("H,G,D,E,window,keep", [(4, 2, 16, 16, 9, 2), (3, 3, 20, 8, 5, 0), (8, 4, 40, 24, 40, 3),
                                                  (2, 1, 8, 8, None, 0), (6, 2, 24, 24, 1, 1)])
 def test_sigmoid_attention_paged(dev, H, G, D, E, window, keep):
     """Ragged batch on scattered pages -- a decode-form sequence, a portion of a prompt behind cached context, a
@@ -146,7 +146,7 @@ def test_sigmoid_attention_paged(dev, H, G, D, E, window, keep):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,G,D,E,window,keep,bs", [(8, 2, 48, 48, 72, 6, 16), (16, 4, 64, 64, 40, 3, 16),
+@pytest.mark.parametrize("H,G,D,E,window,keep,bs", [(8, 2, 40, 56, 70, 5, 16), (16, 4, 64, 64, 40, 3, 16),
                                                     (4, 4, 128, 128, None, 0, 32), (16, 16, 32, 104, 300, 2, 16),
                                                     (3, 1, 24, 8, 33, 40, 8)])
 def test_sigmoid_attention_matrix_core_form(monkeypatch, H, G, D, E, window, keep, bs):

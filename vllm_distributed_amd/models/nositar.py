@@ -138,8 +138,6 @@ class NositarForCausalLM(nn.Module):
         cap = config.get("logit_softcap")
         self.soft_cap = float(cap) if cap else None
         self.logits_processor = LogitsProcessor(int(config.vocab))
-        self.keep_layer_outputs = False          # debugging aid: sum of the streams after every layer
-        self.layer_outputs: list[torch.Tensor] = []
 
     def get_input_embeddings(self, input_ids):
         return self.embed_tokens(input_ids) * self.embed_scale
@@ -152,12 +150,9 @@ class NositarForCausalLM(nn.Module):
             xs = ops.stream_embed(input_ids, self.embed_tokens.weight, self.embed_scale, self.streams)
         n = len(self.layers)
         h = read_streams(xs, self.layers[0].port1, self.layers[0].norm1, dtype) if n else None
-        self.layer_outputs = []
         for i, layer in enumerate(self.layers):
             nxt = self.layers[i + 1] if i + 1 < n else None
             h = layer(xs, h, nxt.port1 if nxt else self.out_port, nxt.norm1 if nxt else self.norm)
-            if self.keep_layer_outputs:
-                self.layer_outputs.append(xs.sum(0))
         return h if n else read_streams(xs, self.out_port, self.norm, dtype)
 
     def compute_logits(self, hidden_states):

@@ -99,9 +99,6 @@ def ensure_built_for(model_dir: str | None, log=None) -> None:
         return
     only = None
     try:
-        import json
-        with open(os.path.join(model_dir, "config.json")) as f:
-            d = json.load(f)
         from ..config import load_hf_config
         from ..models.registry import ModelRegistry
         cls, _ = ModelRegistry.resolve_model_cls(list(load_hf_config(model_dir).get("architectures") or []))

@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void sigmoid_window_attention_kernel(
 //      keys (8 (lane >> 4) ..) of every head, in registers;
 //   2. the same wave mixes them over heads (fp32, weights from LDS), adds the bias, applies the sigmoid and the
 //      visibility, and leaves the 8 weights of every head as one 16-byte row in LDS -- already in the layout of an
-//      MFMA B operand;
+//      MFMA B operand (the mixing weights sit in LDS too: one broadcast read per four heads);
 //   3. after a barrier the waves change roles: wave w owns heads [w H/4, (w+1) H/4) and accumulates
 //      O^T += V^T . P^T over the four 32-key parts (A = value rows with 8 contiguous keys, which is what the
 //      cache's V layout stores).
@@ -205,7 +205,9 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
   using V8 = typename Vec<T>::v8;
   constexpr int HPW = MAXH / 4;                 // heads a wave accumulates
   extern __shared__ __align__(16) unsigned char smem[];
-  V8* pl = reinterpret_cast<V8*>(smem);         // [MAXH][4][64] weights, 16 bytes each: the whole LDS footprint
+  V8* pl = reinterpret_cast<V8*>(smem);         // [MAXH][4][64] weights, 16 bytes each
+  float* tk = reinterpret_cast<float*>(smem + (size_t)MAXH * 4 * 64 * 16);    // [MAXH][MAXH] mixing weights x scale
+  float* pbs = tk + MAXH * MAXH;                                              // [MAXH]
 
   const int s = blockIdx.y, tid = threadIdx.x;
   const int sl = seq_lens[s];
@@ -220,6 +222,12 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
   const int nblk = (sl + bs - 1) / bs;
   const int lane = tid & 63, wave = tid >> 6, r = lane & 15, g4 = lane >> 4;
 
+  for (int e = tid; e < MAXH * MAXH; e += 256) {
+    const int hh = e / MAXH, gg = e % MAXH;
+    tk[e] = (hh < H && gg < H) ? talk[hh * H + gg] * scale : 0.f;
+  }
+  for (int e = tid; e < MAXH; e += 256) pbs[e] = e < H ? pb[e] : 0.f;
+  __syncthreads();
   // this lane's query row (columns beyond the tile repeat the last one; they are masked and never stored)
   const T* qrow = qn + (long)(t0 + i0 + min(r, nq - 1)) * H * D;
   V8 zero8;
@@ -294,16 +302,16 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(
       for (int h = 0; h < MAXH; ++h) {
         if (h < H) {
           float m[8];
-          const float bias = pb[h];
+          const float bias = pbs[h];
 #pragma unroll
           for (int j = 0; j < 8; ++j) m[j] = bias;
 #pragma unroll
-          for (int g = 0; g < MAXH; ++g) {
-            if (g < H) {                       // uniform: the mixing weight comes through the scalar unit
-              const float w = talk[h * H + g] * scale;
+          for (int g4i = 0; g4i < MAXH / 4; ++g4i) {          // one broadcast 16-byte LDS read per four heads
+            const f32x4 w4 = *reinterpret_cast<const f32x4*>(tk + h * MAXH + 4 * g4i);
 #pragma unroll
-              for (int j = 0; j < 8; ++j) m[j] += w * raw[g][j];
-            }
+            for (int gg = 0; gg < 4; ++gg)
+#pragma unroll
+              for (int j = 0; j < 8; ++j) m[j] += w4[gg] * raw[4 * g4i + gg][j];
           }
           V8 pv;
 #pragma unroll
@@ -389,7 +397,7 @@ static int launch_sigmoid_mfma(dim3 grid, hipStream_t st, void* out, const void*
                                const int* qsl, const float* talk, const float* pb, float scale, int window,
                                int keep_first, int H, int G, int D, int Dv, int bs, float* part, long part_stride) {
   const int MAXH = H <= 8 ? 8 : 16, KS = D <= 64 ? 2 : 4, NT = Dv <= 64 ? 4 : 8;
-  const size_t lds = (size_t)MAXH * 4 * 64 * 16;
+  const size_t lds = (size_t)MAXH * 4 * 64 * 16 + ((size_t)MAXH * MAXH + MAXH) * 4;
 #define LM(MH, KK, NN)                                                                                              \
   do {                                                                                                              \
     if (lds > 48 * 1024) {                                                                                          \
