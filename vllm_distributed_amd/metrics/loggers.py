@@ -94,7 +94,9 @@ class PrometheusStatLogger(StatLoggerBase):
             try:
                 m = kind(name, doc, labelnames=names, **kw)
             except ValueError:      # already registered in this process (several engines / tests)
-                m = pc.REGISTRY._names_to_collectors[name.removesuffix("_total")]
+                # counters are registered without their "_total"; a histogram whose own name ends in it is not
+                known = pc.REGISTRY._names_to_collectors
+                m = known[name] if name in known else known[name.removesuffix("_total")]
             return m.labels(**labels)
 
         G, C, H = pc.Gauge, pc.Counter, pc.Histogram
