@@ -167,6 +167,9 @@ def load_hf_config(model: str, overrides: Optional[dict] = None) -> HFConfig:
     if d.get("architecture") == "Nositar":         # a layer-list configuration with names of its own
         from .models.nositar import normalise_config as nositar_config
         d = nositar_config(d, model if os.path.isdir(model) else None)
+    if d.get("architecture") == "Rapovik":         # likewise, with a loop over part of the layers
+        from .models.rapovik import normalise_config as rapovik_config
+        d = rapovik_config(d, model if os.path.isdir(model) else None)
     if d.get("model_type") in ("exaone", "telechat", "qwen", "chatglm"):
         from .models.renamed_decoders import normalise_config
         d = normalise_config(d)
@@ -334,7 +337,7 @@ class ModelConfig:
                          # encoder-decoder: the cross-attention cache is per-request state of the same kind
                          "WhisperForConditionalGeneration", "BartForConditionalGeneration", "BartModel",
                          "MllamaForConditionalGeneration", "Zamba2ForCausalLM", "Plamo2ForCausalLM",
-                         "Florence2ForConditionalGeneration", "NositarForCausalLM")
+                         "Florence2ForConditionalGeneration", "NositarForCausalLM", "RapovikForCausalLM")
                    for a in self.architectures)
 
     @property

@@ -456,9 +456,18 @@ class MLAAttention(nn.Module):
     """
     is_mla = True
 
-    def __init__(self, num_heads: int, kv_lora_rank: int, rope_dim: int, scale: float, prefix: str = ""):
+    def __init__(self, num_heads: int, kv_lora_rank: int, rope_dim: int, scale: float, prefix: str = "",
+                 sliding_window: int = 0, transposed_copy: bool = True):
         super().__init__()
         self.num_heads, self.kv_lora_rank, self.rope_dim = num_heads, kv_lora_rank, rope_dim
+        # > 0: position i sees the keys j with 0 <= i - j < sliding_window.  The pages of hidden keys stay with the
+        # request (a full-attention layer to the cache manager); the kernel never loads them.
+        self.sliding_window = int(sliding_window or 0)
+        # False: the cache keeps the latent rows only and ``forward_cached`` attends over them with the kernel for
+        # any sizes and windows (ops.latent_window_attention); the caller writes the rows itself
+        self.transposed_copy = bool(transposed_copy)
+        if self.sliding_window and self.transposed_copy:
+            raise ValueError("windowed latent attention runs on the rows-only cache (transposed_copy=False)")
         self.dk, self.dv = kv_lora_rank + rope_dim, kv_lora_rank
         self.scale = float(scale)
         self.layer_name = prefix
@@ -472,7 +481,7 @@ class MLAAttention(nn.Module):
     def get_kv_cache_spec(self, block_size: int, dtype: torch.dtype) -> KVCacheSpec:
         # fp8: e4m3 bytes of value / _kv_scale_float (normalised latents and rotated keys sit well inside its range)
         return MLASpec(block_size=block_size, num_kv_heads=1, head_size=self.dk, dtype=dtype, use_mla=True,
-                       v_size=self.dv)
+                       v_size=self.dv if self.transposed_copy else 0)
 
     def bind_kv_cache(self, k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
         self.k_cache, self.v_cache = k_cache, v_cache
@@ -498,4 +507,20 @@ class MLAAttention(nn.Module):
             nsplit = ops.decode_num_splits(S * max(self.num_heads // 16, 1), 1, self.max_model_len)
         ops.mla_attention(out[:n], q[:n], self.k_cache, self.v_cache, md.block_table[:S], md.seq_lens[:S],
                           md.query_start_loc[:S + 1], self.scale, md.max_query_len, nsplit, self._kv_scale_float)
+        return out
+
+    def forward_cached(self, q: torch.Tensor) -> torch.Tensor:
+        """Attention over rows the caller has already written to ``k_cache`` for this step's tokens (rows-only
+        cache).  q [T, H, dk]; returns [T, H, kv_lora_rank]."""
+        md: Optional[AttentionMetadata] = get_forward_context().attn_metadata
+        T = q.shape[0]
+        if md is None or self.k_cache is None:
+            return torch.zeros((T, self.num_heads, self.dv), dtype=q.dtype, device=q.device)
+        n = md.num_actual_tokens
+        S = md.num_decode_seqs + md.num_prefill_seqs
+        out = ops.latent_window_attention(q[:n], self.k_cache, md.block_table[:S], md.seq_lens[:S],
+                                          md.query_start_loc[:S + 1], self.scale, self.sliding_window, self.dv,
+                                          md.max_query_len)
+        if n < T:
+            out = torch.cat([out, out.new_zeros((T - n, self.num_heads, self.dv))], dim=0)
         return out

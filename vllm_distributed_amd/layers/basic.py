@@ -89,6 +89,17 @@ class MulAndSilu(nn.Module):
         return ops.act_and_mul(x, "silu", act_first=False)
 
 
+class ClampedSwigluAndMul(nn.Module):
+    """[gate | up] -> g * sigmoid(1.702 g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)."""
+
+    def __init__(self, limit: float):
+        super().__init__()
+        self.limit = float(limit)
+
+    def forward(self, x):
+        return ops.act_and_mul(x, "clamped_swiglu", threshold=self.limit)
+
+
 class FatreluAndMul(nn.Module):
     def __init__(self, threshold: float = 0.0):
         super().__init__()

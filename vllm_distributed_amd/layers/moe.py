@@ -49,7 +49,7 @@ def grouped_topk(scores: torch.Tensor, k: int, renormalize: bool, num_expert_gro
     T, E = scores.shape
     sel = scores + bias.unsqueeze(0) if bias is not None else scores
     g = sel.view(T, num_expert_group, -1)
-    gscore = g.topk(2, dim=-1)[0].sum(-1) if bias is not None else g.max(dim=-1).values
+    gscore = g.topk(min(2, g.shape[-1]), dim=-1)[0].sum(-1) if bias is not None else g.max(dim=-1).values
     gidx = gscore.topk(topk_group, dim=-1, sorted=False)[1]
     gmask = torch.zeros_like(gscore).scatter_(1, gidx, 1.0)
     mask = gmask.unsqueeze(-1).expand(T, num_expert_group, E // num_expert_group).reshape(T, E)
@@ -75,7 +75,8 @@ class UnquantizedMoEMethod:
 
     def apply(self, layer: "FusedMoE", x: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor) -> torch.Tensor:
         return ops.fused_moe(x, layer.w13_weight, layer.w2_weight, topk_w, topk_ids,
-                             activation=getattr(layer, "activation", "silu"))
+                             activation=getattr(layer, "activation", "silu"),
+                             act_limit=getattr(layer, "act_limit", 0.0))
 
 
 class FusedMoE(nn.Module):
@@ -87,12 +88,13 @@ class FusedMoE(nn.Module):
                  topk_group: Optional[int] = None, quant_config=None, prefix: str = "",
                  custom_routing_function: Optional[Callable] = None, scoring_func: str = "softmax",
                  e_score_correction_bias: Optional[torch.Tensor] = None, routed_scaling_factor: float = 1.0,
-                 activation: str = "silu"):
+                 activation: str = "silu", act_limit: float = 0.0):
         super().__init__()
         if activation not in ops.MOE_ACTIVATIONS:
             raise ValueError(f"{prefix}: expert activation {activation!r} is not supported "
                              f"(supported: {', '.join(ops.MOE_ACTIVATIONS)})")
         self.activation = activation            # of the gate half, fused into the first expert GEMM
+        self.act_limit = float(act_limit)       # the clamp of activations that have one ("clamped_swiglu")
         self.params_dtype = params_dtype or torch.get_default_dtype()
         self.global_num_experts, self.top_k = num_experts, top_k
         self.hidden_size = hidden_size

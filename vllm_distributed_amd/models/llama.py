@@ -18,7 +18,7 @@ import torch.nn as nn
 
 from ..config import VllmConfig
 from ..layers.attention import Attention
-from ..layers.basic import (GemmaRMSNorm, LogitsProcessor, ParallelLMHead, RMSNorm, SiluAndMul, VocabParallelEmbedding,
+from ..layers.basic import (ClampedSwigluAndMul, GemmaRMSNorm, LogitsProcessor, ParallelLMHead, RMSNorm, SiluAndMul, VocabParallelEmbedding,
                             get_act_and_mul_fn)
 from ..forward_context import get_forward_context, has_forward_context
 from ..layers.linear import (MergedColumnParallelLinear, QKVParallelLinear, RowParallelLinear,
@@ -32,13 +32,14 @@ from .utils import (IntermediateTensors, PPMissingLayer, load_weights_with_mappi
 
 class LlamaMLP(nn.Module):
     def __init__(self, hidden_size: int, intermediate_size: int, bias: bool = False, quant_config=None,
-                 prefix: str = "", reduce_results: bool = True, act: str = "silu"):
+                 prefix: str = "", reduce_results: bool = True, act: str = "silu", act_limit: float = 0.0):
         super().__init__()
         self.gate_up_proj = MergedColumnParallelLinear(hidden_size, [intermediate_size] * 2, bias=bias,
                                                        quant_config=quant_config, prefix=f"{prefix}.gate_up_proj")
         self.down_proj = RowParallelLinear(intermediate_size, hidden_size, bias=bias, quant_config=quant_config,
                                            reduce_results=reduce_results, prefix=f"{prefix}.down_proj")
-        self.act_fn = SiluAndMul() if act == "silu" else get_act_and_mul_fn(act)
+        self.act_fn = SiluAndMul() if act == "silu" else ClampedSwigluAndMul(act_limit) if act == "clamped_swiglu" \
+            else get_act_and_mul_fn(act)
         self._silu = act == "silu"
 
     def forward(self, x):

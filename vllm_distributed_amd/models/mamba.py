@@ -62,11 +62,55 @@ class StateSpaceLayer(nn.Module):
 
     def bind_kv_cache(self, conv_state: torch.Tensor, ssm_state: torch.Tensor) -> None:
         self.conv_state, self.ssm_state = conv_state, ssm_state
+        self._first_pass = (conv_state, ssm_state)
 
     @staticmethod
     def slot_table(md) -> torch.Tensor:
         """[S, >=1] int32 whose column 0 is each sequence's state slot."""
         return md.state_table if md.state_table is not None else md.block_table
+
+    # A stack that runs a layer several times with the same weights keeps one state per pass: the mixer owns the
+    # first, a ``PassState`` child each further one, and the model names the pass before it calls the mixer.
+    def add_passes(self, passes: int) -> None:
+        self.pass_states = nn.ModuleList([PassState(self) for _ in range(passes - 1)])
+
+    def select_pass(self, index: int) -> None:
+        if index == 0:
+            self.conv_state, self.ssm_state = getattr(self, "_first_pass", (self.conv_state, self.ssm_state))
+        else:
+            st = self.pass_states[index - 1]
+            self.conv_state, self.ssm_state = st.conv_state, st.ssm_state
+
+
+class PassState(nn.Module):
+    """State tensors of one further pass over a mixer (same shapes and types as the mixer's own)."""
+    is_state_space_layer = True
+
+    def __init__(self, owner: StateSpaceLayer):
+        super().__init__()
+        self._owner = [owner]                  # in a list: the owner is not a submodule of its own child
+        self.conv_state: Optional[torch.Tensor] = None
+        self.ssm_state: Optional[torch.Tensor] = None
+        self.layer_name = ""
+
+    @property
+    def conv_dtype(self):
+        return self._owner[0].conv_dtype
+
+    @property
+    def state_dtypes(self):
+        o = self._owner[0]
+        return getattr(o, "state_dtypes", (o.conv_dtype, torch.float32))
+
+    def state_shapes(self) -> tuple:
+        return self._owner[0].state_shapes()
+
+    def get_kv_cache_spec(self, block_size: int, dtype: torch.dtype) -> KVCacheSpec:
+        return MambaSpec(block_size=self._owner[0].max_model_len, shapes=self.state_shapes(),
+                         dtypes=tuple(self.state_dtypes))
+
+    def bind_kv_cache(self, conv_state: torch.Tensor, ssm_state: torch.Tensor) -> None:
+        self.conv_state, self.ssm_state = conv_state, ssm_state
 
 
 class MambaMixer(StateSpaceLayer):
@@ -154,6 +198,11 @@ class Mamba2Mixer(StateSpaceLayer):
         if self.d_inner != self.num_heads * self.head_dim:
             self.d_inner = self.num_heads * self.head_dim
         self.d_state = int(config.state_size)
+        # the scan kernel is built for states of 16, 32, ... 256 values: other widths run zero-padded to the next of
+        # these (padded B columns keep their state entries at zero, padded C columns read nothing)
+        self.d_state_padded = next((n for n in (16, 32, 64, 128, 256) if n >= self.d_state), None)
+        if self.d_state_padded is None:
+            raise ValueError(f"{prefix}: state size {self.d_state} is beyond the scan kernel (at most 256)")
         self.d_conv = int(config.conv_kernel)
         self.n_groups = int(config.n_groups)
         self.conv_dim = self.d_inner + 2 * self.n_groups * self.d_state
@@ -188,7 +237,7 @@ class Mamba2Mixer(StateSpaceLayer):
         self.out_proj = RowParallelLinear(self.d_inner, self.hidden, bias=use_bias, prefix=f"{prefix}.out_proj")
 
     def state_shapes(self) -> tuple:
-        return ((self.conv_dim, self.d_conv - 1), (self.d_inner, self.d_state))
+        return ((self.conv_dim, self.d_conv - 1), (self.d_inner, self.d_state_padded))
 
     def _gated_norm(self, y: torch.Tensor) -> torch.Tensor:
         # y already carries the silu(gate) factor (applied inside the scan kernel)
@@ -211,6 +260,10 @@ class Mamba2Mixer(StateSpaceLayer):
                                 md.seq_lens, tbl, md.max_query_len)
         gn = self.n_groups * self.d_state
         xs, B, C = xbc[:, :di], xbc[:, di:di + gn], xbc[:, di + gn:]
+        if self.d_state_padded != self.d_state:
+            pad, T = self.d_state_padded - self.d_state, xbc.shape[0]
+            B = torch.nn.functional.pad(B.reshape(T, self.n_groups, self.d_state), (0, pad)).reshape(T, -1)
+            C = torch.nn.functional.pad(C.reshape(T, self.n_groups, self.d_state), (0, pad)).reshape(T, -1)
         bias, softplus = self.dt_bias, True
         if self.dt_limit is not None:
             dt = torch.nn.functional.softplus(dt.float() + self.dt_bias).clamp(*self.dt_limit).to(x.dtype)

@@ -115,7 +115,7 @@ def layer_norm(x, weight, bias, eps):
 def act_and_mul(x, kind: str = "silu", act_first: bool = True, threshold: float = 0.0,
                 out: Optional[torch.Tensor] = None, fp8_scale: Optional[torch.Tensor] = None):
     d = x.shape[-1] // 2
-    if not _dev(x):
+    if not _dev(x) or d % 8:
         y = R.act_and_mul(x, kind, act_first, threshold)
         if fp8_scale is not None:
             y = R.scaled_fp8_quant(y, fp8_scale)[0]
@@ -916,7 +916,7 @@ def fp8_gemm(xq: torch.Tensor, w: torch.Tensor, x_scale: torch.Tensor, w_scale: 
     out = torch.empty((M, N_), dtype=out_dtype, device=xq.device)
     N.call("vda_tile_gemm", out.data_ptr(), xq.data_ptr(), w.data_ptr(), xs.data_ptr(), ws.data_ptr(), None,
            N.ptr(bias), None, None, None, None, None, M, N_, K, 1, 0, xq.stride(0), out.stride(0), 0, EPI_PLAIN,
-           SC_BLOCK if block else SC_TOKEN, _tile_rows(M), N.dt(xq.dtype), N.dt(out_dtype), 0, N.stream())
+           SC_BLOCK if block else SC_TOKEN, _tile_rows(M), N.dt(xq.dtype), N.dt(out_dtype), 0, 0.0, N.stream())
     return out
 
 
@@ -978,7 +978,7 @@ def tile_linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     out = torch.empty((M, N_), dtype=x.dtype, device=x.device)
     N.call("vda_tile_gemm", out.data_ptr(), x.data_ptr(), w.data_ptr(), None, None, None, N.ptr(bias), None, None,
            None, None, None, M, N_, K, 1, 0, x.stride(0), out.stride(0), 0, EPI_PLAIN, SC_NONE,
-           rows_per_tile or _tile_rows(M), N.dt(x.dtype), N.dt(x.dtype), 0, N.stream())
+           rows_per_tile or _tile_rows(M), N.dt(x.dtype), N.dt(x.dtype), 0, 0.0, N.stream())
     return out
 
 
@@ -1007,7 +1007,7 @@ def moe_align_tiles(topk_ids: torch.Tensor, E: int, rows_per_tile: int):
 
 
 def _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales: bool = False,
-               activation: str = "silu", x_scale=None, out_dtype=None):
+               activation: str = "silu", x_scale=None, out_dtype=None, act_limit: float = 0.0):
     """Compute-bound batches: both expert GEMMs run as LDS-tiled MFMA GEMMs over the expert-sorted pairs
     (ops/csrc/gemm_tile.hip).  e4m3 weights: activations are quantised per token (or per group of 128
     with block-scaled weights) and the fp8 matrix cores do the products; 16-bit weights: 16-bit MFMA.
@@ -1041,7 +1041,8 @@ def _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales: 
         mode, xq, xs = SC_NONE, _contig_last(x), None
     N.call("vda_tile_gemm", inter.data_ptr(), xq.data_ptr(), w13.data_ptr(), N.ptr(xs), N.ptr(w13_scale), None, None,
            sorted_ids.data_ptr(), te.data_ptr(), tb.data_ptr(), tend.data_ptr(), ntl.data_ptr(), 0, I, H, k,
-           max_tiles, xq.stride(0), I, I2 * H, EPI_GATE_UP, mode, rows, N.dt(xq.dtype), N.dt(odt), N.ACT[activation], st)
+           max_tiles, xq.stride(0), I, I2 * H, EPI_GATE_UP, mode, rows, N.dt(xq.dtype), N.dt(odt), N.ACT[activation],
+           float(act_limit), st)
     if fp8:
         hq, hs = per_group_fp8_quant(inter) if block_scales else per_token_fp8_quant(inter)
         hs = hs.contiguous()
@@ -1050,7 +1051,7 @@ def _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales: 
     N.call("vda_tile_gemm", out2.data_ptr(), hq.data_ptr(), w2.data_ptr(), N.ptr(hs), N.ptr(w2_scale),
            tw.data_ptr(), None, sorted_ids.data_ptr(), te.data_ptr(), tb.data_ptr(), tend.data_ptr(),
            ntl.data_ptr(), 0, H, I, 1, max_tiles, hq.stride(0), H, H * I, EPI_DOWN, mode, rows, N.dt(hq.dtype),
-           N.dt(odt), 0, st)
+           N.dt(odt), 0, 0.0, st)
     N.call("vda_moe_sum", out.data_ptr(), out2.data_ptr(), topk_ids.contiguous().data_ptr(), T, H, k,
            out.stride(0), N.dt(odt), st)
     return out
@@ -1097,13 +1098,13 @@ def moe_rows_form(num_pairs: int, num_experts: int, rows: int, weight_bytes: int
     return wide if avg >= 8 and (fills or avg >= 64) else 0
 
 
-MOE_ACTIVATIONS = ("silu", "gelu", "gelu_tanh", "gelu_pytorch_tanh", "relu", "relu2")
+MOE_ACTIVATIONS = ("silu", "gelu", "gelu_tanh", "gelu_pytorch_tanh", "relu", "relu2", "clamped_swiglu")
 
 
 def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor,
               w13_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
               block_scales: bool = False, activation: str = "silu", x_scale: Optional[torch.Tensor] = None,
-              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+              out_dtype: Optional[torch.dtype] = None, act_limit: float = 0.0) -> torch.Tensor:
     """Routed gated expert MLPs, out[t] = sum_j w[t, j] * W2_e(act(Wg_e x_t) * (Wu_e x_t)) with ``activation`` one of
     MOE_ACTIVATIONS (reference: vllm/model_executor/layers/fused_moe/fused_moe.py:1003,1034 ``activation``), fused
     into the first GEMM's epilogue in every kernel form.  x [T,H]; w13 [E,2I,H] (gate rows then up rows); w2 [E,H,I];
@@ -1116,7 +1117,8 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
         # x is e4m3 with one scale per row (see moe_fp8_rows_ok): straight into the fp8 tiles, or widened again
         odt = out_dtype or torch.bfloat16
         if _dev(x) and not block_scales and moe_tiled_ok(torch.empty(0, dtype=odt), w13, w2):
-            return _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, False, activation, x_scale, odt)
+            return _moe_tiled(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, False, activation, x_scale, odt,
+                              act_limit)
         x = (x.float() * x_scale.float().reshape(-1, 1)).to(odt)
     if _dev(x) and block_scales and not moe_tiled_ok(x, w13, w2):
         raise RuntimeError(f"block-scaled expert shapes {tuple(w13.shape)} / {tuple(w2.shape)} are outside the tiled "
@@ -1127,9 +1129,10 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
                 f"expert shapes {tuple(w13.shape)} / {tuple(w2.shape)} are outside the grouped MoE kernel (hidden and "
                 "expert width must be multiples of 128); the PyTorch fallback synchronises and cannot be captured "
                 "into a hipGraph: run with enforce_eager=True")
-        return R.fused_moe(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales, activation)
+        return R.fused_moe(x, w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales, activation, act_limit)
     if not moe_grouped_ok(x, w13, w2):
-        return _moe_tiled(_contig_last(x), w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales, activation)
+        return _moe_tiled(_contig_last(x), w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales, activation,
+                          act_limit=act_limit)
     T, H = x.shape
     k = topk_ids.shape[1]
     E, I2, _ = w13.shape
@@ -1140,7 +1143,8 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
     if w13.dtype == torch.float8_e4m3fn:
         limit = min(limit, envs.VDA_MOE_GROUPED_MAX_PAIRS_FP8)
     if T * k > limit or block_scales:
-        return _moe_tiled(_contig_last(x), w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales, activation)
+        return _moe_tiled(_contig_last(x), w13, w2, topk_w, topk_ids, w13_scale, w2_scale, block_scales, activation,
+                          act_limit=act_limit)
     x = _contig_last(x)
     dev = x.device
     ids = topk_ids.contiguous()
@@ -1157,7 +1161,7 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
     max_pairs = T
     N.call("vda_moe_gate_up", inter.data_ptr(), x.data_ptr(), w13.data_ptr(), N.ptr(w13_scale), sorted_ids.data_ptr(),
            offsets.data_ptr(), E, I, H, k, max_pairs, x.stride(0), N.dt(x.dtype), wd,
-           int(moe_rows_form(T * k, E, I, w13.element_size())), N.ACT[activation], st)
+           int(moe_rows_form(T * k, E, I, w13.element_size())), N.ACT[activation], float(act_limit), st)
     N.call("vda_moe_down", out2.data_ptr(), inter.data_ptr(), w2.data_ptr(), N.ptr(w2_scale), tw.data_ptr(),
            sorted_ids.data_ptr(), offsets.data_ptr(), E, H, I, max_pairs, N.dt(x.dtype), wd,
            int(moe_rows_form(T * k, E, H, w2.element_size())), st)
@@ -1389,4 +1393,91 @@ def gated_delta_rule(qkv: torch.Tensor, a_raw: torch.Tensor, b_raw: torch.Tensor
            gate_raw.stride(0), a_log.data_ptr(), dt_bias.data_ptr(), norm_w.data_ptr(), state.data_ptr(),
            query_start_loc.data_ptr(), seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), T, S, H, G,
            D, Dv, float(eps), N.dt(qkv.dtype), N.stream())
+    return out
+
+
+# ---- fp32 residual with a norm after and before every sub-layer ------------------------------------------------
+def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, w_post: Optional[torch.Tensor] = None,
+                   w_pre: Optional[torch.Tensor] = None, eps: float = 1e-6, out_dtype: Optional[torch.dtype] = None,
+                   gain_offset: float = 1.0) -> Optional[torch.Tensor]:
+    """One pass over the fp32 residual ``x`` [T, W]: with ``y`` (a sub-layer's output) x += y / rms(y) *
+    (gain_offset + w_post), in place; with ``w_pre`` returns x / rms(x) * (gain_offset + w_pre) in ``out_dtype``
+    (the next sub-layer's input).  Gains are fp32 tensors [W]."""
+    T, W = x.shape
+    if not _dev(x) or W * 4 > 60 * 1024:
+        return R.residual_norms(x, y, w_post, w_pre, eps, out_dtype, gain_offset)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    h = torch.empty((T, W), dtype=out_dtype, device=x.device) if w_pre is not None else None
+    if y is not None:
+        assert y.stride(1) == 1 and y.shape == (T, W) and w_post.dtype == torch.float32
+        assert h is None or h.dtype == y.dtype
+    N.call("vda_residual_norms", x.data_ptr(), N.ptr(y), y.stride(0) if y is not None else 0, N.ptr(w_post),
+           N.ptr(w_pre), N.ptr(h), W, float(eps), float(gain_offset), T, W,
+           N.dt(y.dtype if y is not None else h.dtype), N.stream())
+    return h
+
+
+# ---- latent attention over a window -----------------------------------------------------------------------------
+def latent_norm_rope_cache(q: torch.Tensor, down: torch.Tensor, c_weight: torch.Tensor, cos_sin: torch.Tensor,
+                           positions: torch.Tensor, qf: torch.Tensor, kc: Optional[torch.Tensor],
+                           slot_mapping: torch.Tensor, H: int, D: int, P: int, rank: int, rot_dims: int,
+                           eps: float) -> None:
+    """Per token: the cache row [down[:rank] / rms * c_weight | down[rank:] with its first ``rot_dims`` values rotated] goes
+    to ``kc`` [blocks, bs, rank + P] at ``slot_mapping``; the last P values of every query head (q [T, H * (D + P)]),
+    rotated alike, go to qf[:, h, rank:] (qf [T, H, rank + P]).  Pairs (2i, 2i + 1) turn by the angle whose cosine and sine
+    are cos_sin[position, i] and cos_sin[position, rot_dims / 2 + i] (fp32)."""
+    if not _dev(q):
+        return R.latent_norm_rope_cache(q, down, c_weight, cos_sin, positions, qf, kc, slot_mapping, H, D, P, rank,
+                                        rot_dims, eps)
+    T = q.shape[0]
+    assert q.stride(1) == 1 and down.stride(1) == 1 and qf.is_contiguous() and kc.is_contiguous()
+    assert q.dtype == down.dtype == qf.dtype == kc.dtype and kc.shape[2] == rank + P and qf.shape == (T, H, rank + P)
+    assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == max(rot_dims, 1)
+    assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int64 and c_weight.dtype == torch.float32
+    N.call("vda_latent_norm_rope_cache", q.data_ptr(), q.stride(0), down.data_ptr(), down.stride(0),
+           c_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(), qf.data_ptr(), kc.data_ptr(),
+           slot_mapping.data_ptr(), T, H, D, P, rank, rot_dims, kc.shape[1], float(eps), N.dt(q.dtype), N.stream())
+
+
+def latent_window_attention(q: torch.Tensor, kc: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,
+                            query_start_loc: torch.Tensor, scale: float, window: int, rank: int,
+                            max_query_len: int) -> torch.Tensor:
+    """Softmax attention of q [T, H, DK] over the latent rows kc [blocks, bs, DK] of each sequence's visible keys
+    (j <= i, and i - j < window when window > 0); returns the weighted sums of the rows' first ``rank`` values [T, H, rank]."""
+    if not _dev(q):
+        return R.latent_window_attention(q, kc, block_table, seq_lens, query_start_loc, scale, window, rank)
+    T, H, DK = q.shape
+    assert q.is_contiguous() and kc.is_contiguous() and kc.dtype == q.dtype and kc.shape[2] == DK
+    out = torch.zeros((T, H, rank), dtype=q.dtype, device=q.device)
+    N.call("vda_latent_window_attention", out.data_ptr(), q.data_ptr(), kc.data_ptr(), block_table.data_ptr(),
+           block_table.stride(0), seq_lens.data_ptr(), query_start_loc.data_ptr(), float(scale), int(window),
+           seq_lens.shape[0], H, DK, rank, kc.shape[1], max(int(max_query_len), 1), N.dt(q.dtype), N.stream())
+    return out
+
+
+# ---- matrix memory with exponential gates (mLSTM) ----------------------------------------------------------------
+def mlstm(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, norm_w: torch.Tensor,
+          state_nm: torch.Tensor, state_s: torch.Tensor, query_start_loc: torch.Tensor, seq_lens: torch.Tensor,
+          slot_table: torch.Tensor, H: int, D: int, Dv: int, cap: float, eps: float) -> torch.Tensor:
+    """mLSTM cell over a ragged batch (see ops/csrc/mlstm.hip).  proj [T, 2*H*D + 2*H*Dv + 2*H] = [q | k | v | output
+    gate | input gate | forget gate] pre-activations; i_bias, f_bias [H] and norm_w [H * Dv] fp32; state_nm fp32
+    [slots, H, Dn] (n, then the running maximum at [D]) and state_s fp32 [slots, H, D, Dv], updated in place; sequence
+    s uses slot ``slot_table[s, 0]`` and starts from zero when all its tokens are in this batch.
+    Returns [T, H * Dv]: the read-out, normalised per head, times norm_w, times sigmoid(output gate)."""
+    if not _dev(proj):
+        return R.mlstm(proj, i_bias, f_bias, norm_w, state_nm, state_s, query_start_loc, seq_lens, slot_table, H, D,
+                       Dv, cap, eps)
+    T = proj.shape[0]
+    assert proj.stride(1) == 1 and proj.shape[1] == 2 * H * D + 2 * H * Dv + 2 * H
+    assert state_nm.dtype == torch.float32 and state_s.dtype == torch.float32
+    assert state_nm.is_contiguous() and state_s.is_contiguous() and state_s.shape[1:] == (H, D, Dv)
+    assert state_nm.shape[1] == H and state_nm.shape[2] >= D + 1
+    for t in (i_bias, f_bias, norm_w):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    out = torch.empty((T, H * Dv), dtype=proj.dtype, device=proj.device)
+    o_raw = torch.zeros((T, H * Dv), dtype=torch.float32, device=proj.device)
+    N.call("vda_mlstm", out.data_ptr(), out.stride(0), o_raw.data_ptr(), proj.data_ptr(), proj.stride(0),
+           i_bias.data_ptr(), f_bias.data_ptr(), norm_w.data_ptr(), state_nm.data_ptr(), state_s.data_ptr(),
+           query_start_loc.data_ptr(), seq_lens.data_ptr(), slot_table.data_ptr(), slot_table.stride(0), T,
+           seq_lens.shape[0], H, D, Dv, state_nm.shape[2], float(cap), float(eps), N.dt(proj.dtype), N.stream())
     return out

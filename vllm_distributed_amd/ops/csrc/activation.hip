@@ -3,7 +3,8 @@
 #include "common.h"
 
 enum Act { ACT_SILU = 0, ACT_GELU = 1, ACT_GELU_TANH = 2, ACT_RELU = 3, ACT_GELU_NEW = 4,
-           ACT_GELU_FAST = 5, ACT_GELU_QUICK = 6, ACT_FATRELU = 7, ACT_RELU2 = 8 };
+           ACT_GELU_FAST = 5, ACT_GELU_QUICK = 6, ACT_FATRELU = 7, ACT_RELU2 = 8,
+           ACT_CLAMPED_SWIGLU = 9 /* gated pairs only: see gated_pair, the threshold is its clamp */ };
 
 template <int A> __device__ __forceinline__ float act(float x, float thr) {
   if (A == ACT_SILU) return x / (1.f + __expf(-x));
@@ -40,7 +41,7 @@ __global__ __launch_bounds__(256) void act_and_mul_kernel(void* __restrict__ out
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const float x = (float)a[j], g = (float)b[j];
-      y[j] = ACT_FIRST ? act<A>(x, thr) * g : x * act<A>(g, thr);
+      y[j] = A == ACT_CLAMPED_SWIGLU ? gated_pair(x, g, 9, thr) : ACT_FIRST ? act<A>(x, thr) * g : x * act<A>(g, thr);
     }
     if (QUANT == 0) {
       V8 o;
@@ -87,6 +88,7 @@ static int launch_gated(void* out, const void* in, long rows, int d, long is, lo
       case ACT_GELU_TANH: BYQ(ACT_GELU_TANH, true); break;
       case ACT_FATRELU: BYQ(ACT_FATRELU, true); break;
       case ACT_RELU: BYQ(ACT_RELU, true); break;
+      case ACT_CLAMPED_SWIGLU: BYQ(ACT_CLAMPED_SWIGLU, true); break;
       default: return -2;
     }
   } else {

@@ -169,5 +169,16 @@ __device__ __forceinline__ float gate_act(float x, int kind) {
   }
 }
 
+// A gated pair act(gate) * up with the codes of gate_act, plus 9: both halves clamped, a sigmoid-weighted gate and the
+// up half shifted by one:  g' = min(g, L), u' = clamp(u, -L, L), y = g' * sigmoid(1.702 g') * (u' + 1).
+__device__ __forceinline__ float gated_pair(float g, float u, int kind, float limit) {
+  if (kind == 9) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + __expf(-1.702f * g)) * (u + 1.f);
+  }
+  return gate_act(g, kind) * u;
+}
+
 #define VDA_CHECK_LAUNCH() \
   do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)

@@ -194,3 +194,62 @@ VDA_EXPORT int vda_layer_norm(void* out, const void* in, const void* w, const vo
   VDA_CHECK_LAUNCH();
   return 0;
 }
+
+// ---- fp32 residual with a norm after and before every sub-layer ("sandwich" norms) -----------------------------
+//   x += y / rms(y) * (off + w_post)      (y given: the output of the sub-layer that just ran)
+//   h  = x / rms(x) * (off + w_pre)       (h given: the input of the next sub-layer)
+// One pass over the fp32 residual row per token: the write of one sub-layer and the read of the next are one launch,
+// the role add + RMSNorm fusion plays for 16-bit residuals.  Gains are fp32; `off` is 1 for gains stored around zero.
+template <typename T>
+__global__ __launch_bounds__(256) void residual_norms_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                             long y_stride, const float* __restrict__ w_post,
+                                                             const float* __restrict__ w_pre, T* __restrict__ h,
+                                                             long h_stride, float eps, float off, int W) {
+  extern __shared__ float row[];          // the updated residual row
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int tid = threadIdx.x;
+  float* xr = x + t * W;
+  float ry = 0.f;
+  if (y) {
+    float ss = 0.f;
+    for (int c = tid; c < W; c += 256) {
+      const float v = (float)y[t * y_stride + c];
+      ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    ry = 1.f / sqrtf(ss / (float)W + eps);
+  }
+  float sx = 0.f;
+  for (int c = tid; c < W; c += 256) {
+    float v = xr[c];
+    if (y) {
+      v += (float)y[t * y_stride + c] * ry * (off + w_post[c]);
+      xr[c] = v;
+    }
+    row[c] = v;
+    sx += v * v;
+  }
+  if (!h) return;
+  sx = block_sum(sx, red);
+  const float rx = 1.f / sqrtf(sx / (float)W + eps);
+  for (int c = tid; c < W; c += 256) h[t * h_stride + c] = (T)(row[c] * rx * (off + w_pre[c]));
+}
+
+VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const float* w_post, const float* w_pre,
+                                  void* h, long h_stride, float eps, float off, int T, int W, int dtype,
+                                  hipStream_t st) {
+  if (T <= 0 || (!y && !h)) return 0;
+  if ((y && !w_post) || (h && !w_pre)) return -1;
+  const size_t lds = (size_t)W * 4;
+  if (lds > 60 * 1024) return -2;
+#define L(TT) hipLaunchKernelGGL((residual_norms_kernel<TT>), dim3(T), dim3(256), lds, st, x, (const TT*)y, y_stride, \
+                                 w_post, w_pre, (TT*)h, h_stride, eps, off, W)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
+  VDA_CHECK_LAUNCH();
+  return 0;
+}

@@ -23,7 +23,7 @@ BF16, F16, F32, FP8 = 0, 1, 2, 3
 _DT = {torch.bfloat16: BF16, torch.float16: F16, torch.float32: F32, torch.float8_e4m3fn: FP8}
 
 ACT = {"silu": 0, "gelu": 1, "gelu_tanh": 2, "gelu_pytorch_tanh": 2, "relu": 3, "gelu_new": 4,
-       "gelu_fast": 5, "quick_gelu": 6, "gelu_quick": 6, "fatrelu": 7, "relu2": 8}
+       "gelu_fast": 5, "quick_gelu": 6, "gelu_quick": 6, "fatrelu": 7, "relu2": 8, "clamped_swiglu": 9}
 
 P, I, L, F = c_void_p, c_int, c_long, c_float
 _SIGS = {
@@ -58,13 +58,17 @@ _SIGS = {
     "vda_skinny_gemm": [P, P, P, P, P, I, I, I, L, L, L, I, I, P],
     "vda_moe_topk_softmax": [P, P, P, I, I, I, I, L, I, P],
     "vda_moe_align": [P, P, P, I, I, P],
-    "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, P],
+    "vda_residual_norms": [P, P, L, P, P, P, L, F, F, I, I, I, P],
+    "vda_latent_norm_rope_cache": [P, L, P, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "vda_latent_window_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, I, I, P],
+    "vda_mlstm": [P, L, P, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P],
+    "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, F, P],
     "vda_moe_down": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
     "vda_moe_sum": [P, P, P, I, I, I, L, I, P],
     "vda_ep_prep": [P, I, I, I, P, P, P, P, P, P],
     "vda_moe_tile_map": [P, P, P, P, P, I, I, I, P],
     "vda_moe_align_large": [P, P, P, P, P, I, I, P],
-    "vda_tile_gemm": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, L, L, L, I, I, I, I, I, I, P],
+    "vda_tile_gemm": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, L, L, L, I, I, I, I, I, I, F, P],
     "vda_decode_gemm": [P, P, P, P, P, L, I, I, I, L, L, I, P],
     "vda_wq_gemm": [P, P, P, P, P, P, L, I, I, I, I, I, L, L, I, I, I, P],
     "vda_dense_gemm_stamp": [P, P, P, I, I, I, I, P],

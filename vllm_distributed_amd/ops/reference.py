@@ -55,9 +55,17 @@ def _act(kind: str, x: torch.Tensor, threshold: float = 0.0) -> torch.Tensor:
     raise ValueError(f"unknown activation {kind!r}")
 
 
+def clamped_swiglu(g, u, limit: float):
+    """min(g, limit) * sigmoid(1.702 min(g, limit)) * (clamp(u, -limit, limit) + 1)."""
+    g = g.clamp(max=limit)
+    return g * torch.sigmoid(1.702 * g) * (u.clamp(-limit, limit) + 1.0)
+
+
 def act_and_mul(x, kind="silu", act_first=True, threshold=0.0):
     d = x.shape[-1] // 2
     a, b = x[..., :d].float(), x[..., d:].float()
+    if kind == "clamped_swiglu":          # ``threshold`` carries the limit
+        return clamped_swiglu(a, b, threshold).to(x.dtype)
     y = _act(kind, a, threshold) * b if act_first else a * _act(kind, b, threshold)
     return y.to(x.dtype)
 
@@ -369,7 +377,7 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool):
 
 def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor,
               w13_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
-              block_scales: bool = False, activation: str = "silu") -> torch.Tensor:
+              block_scales: bool = False, activation: str = "silu", act_limit: float = 0.0) -> torch.Tensor:
     """out[t] = sum_j topk_w[t, j] * W2_e( act(Wg_e x_t) * (Wu_e x_t) ), e = topk_ids[t, j];
     negative ids (expert on another rank) contribute nothing.  fp32 accumulation.  ``block_scales``:
     the weight scales are per 128 x 128 block instead of per expert."""
@@ -393,7 +401,10 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
             q, s_ = per_group_fp8_quant(xe.to(x.dtype))
             xe = (q.float().view(*s_.shape, -1) * s_.unsqueeze(-1)).view(xe.shape)
         h = xe @ a.t()
-        act = (_act(activation, h[:, :I]) * h[:, I:]).to(x.dtype).float()
+        if activation == "clamped_swiglu":
+            act = clamped_swiglu(h[:, :I], h[:, I:], act_limit).to(x.dtype).float()
+        else:
+            act = (_act(activation, h[:, :I]) * h[:, I:]).to(x.dtype).float()
         if block_scales:
             q, s_ = per_group_fp8_quant(act.to(x.dtype))
             act = (q.float().view(*s_.shape, -1) * s_.unsqueeze(-1)).view(act.shape)
@@ -672,3 +683,115 @@ def gated_delta_rule(qkv, a_raw, b_raw, gate_raw, a_log, dt_bias, norm_w, state,
     o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
     o = o * torch.sigmoid(gate_raw.float().view(T, H, Dv))
     return o.view(T, H * Dv).to(qkv.dtype)
+
+
+# ---- fp32 residual with a norm after and before every sub-layer ---------------------------------------------
+def residual_norms(x, y, w_post, w_pre, eps: float, out_dtype, gain_offset: float = 1.0):
+    """x fp32 [T, W], in place: x += y / rms(y) * (gain_offset + w_post) when ``y`` is given; returns
+    x / rms(x) * (gain_offset + w_pre) in ``out_dtype`` when ``w_pre`` is given."""
+    if y is not None:
+        f = y.float()
+        x += f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + eps) * (gain_offset + w_post.float())
+    if w_pre is None:
+        return None
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (gain_offset + w_pre.float())).to(out_dtype)
+
+
+# ---- latent attention over a window: cache write and attention ----------------------------------------------
+def rotate_interleaved(x, cos, sin):
+    """x [..., 2n] as pairs (x[2i], x[2i+1]) turned by the angles whose cos / sin [..., n] are given (fp32)."""
+    u, v = x[..., 0::2].float(), x[..., 1::2].float()
+    return torch.stack((u * cos - v * sin, v * cos + u * sin), dim=-1).flatten(-2)
+
+
+def latent_norm_rope_cache(q, down, c_weight, cos_sin, positions, qf, kc, slot_mapping, H: int, D: int, P: int,
+                           R: int, rot_dims: int, eps: float):
+    """q [T, H * (D + P)], down [T, R + P]; cos_sin fp32 [positions, rot_dims] (cosines then sines).
+    Cache row of a token = [rms(down[:R]) * c_weight | rotated down[R:]] -> kc [blocks, bs, R + P] at slot_mapping;
+    the rotated last P values of every query head go to qf[:, h, R:] (qf [T, H, R + P])."""
+    T = q.shape[0]
+    cs = cos_sin[positions[:T].long()]
+    half = rot_dims // 2
+    cos, sin = cs[:, :half], cs[:, half:]
+    c = down[:, :R].float()
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * c_weight.float()
+    kr = down[:, R:].float().clone()
+    kr[:, :rot_dims] = rotate_interleaved(kr[:, :rot_dims], cos, sin)
+    qr = q.view(T, H, D + P)[:, :, D:].float().clone()
+    qr[:, :, :rot_dims] = rotate_interleaved(qr[:, :, :rot_dims], cos[:, None], sin[:, None])
+    qf[:, :, R:] = qr.to(qf.dtype)
+    if kc is not None:
+        bs = kc.shape[1]
+        ok = slot_mapping[:T] >= 0
+        sl = slot_mapping[:T][ok].long()
+        kc[sl // bs, sl % bs] = torch.cat([c, kr], -1)[ok].to(kc.dtype)
+
+
+def latent_window_attention(q, kc, block_table, seq_lens, qsl, scale: float, window: int, R: int):
+    """q [T, H, DK] against the latent rows kc [blocks, bs, DK]: softmax over the keys j <= i with i - j < window
+    (window 0: all of them) of scale * q . row; returns the weighted sums of the rows' first R values, [T, H, R]."""
+    T, H, DK = q.shape
+    bs = kc.shape[1]
+    out = torch.zeros((T, H, R), dtype=torch.float32, device=q.device)
+    for s in range(seq_lens.shape[0]):
+        sl = int(seq_lens[s])
+        t0, t1 = int(qsl[s]), int(qsl[s + 1])
+        L = t1 - t0
+        if sl <= 0 or L <= 0:
+            continue
+        nb = -(-sl // bs)
+        rows = kc[block_table[s, :nb].long()].reshape(nb * bs, DK)[:sl].float()
+        sc = torch.einsum("ihd,jd->hij", q[t0:t1].float(), rows) * scale
+        i = torch.arange(sl - L, sl, device=q.device)[:, None]
+        j = torch.arange(sl, device=q.device)[None, :]
+        vis = j <= i
+        if window > 0:
+            vis = vis & (i - j < window)
+        sc = sc.masked_fill(~vis[None], float("-inf"))
+        out[t0:t1] = torch.einsum("hij,jd->ihd", torch.softmax(sc, -1), rows[:, :R])
+    return out.to(q.dtype)
+
+
+# ---- matrix memory with exponential gates and a running maximum (mLSTM) --------------------------------------
+def mlstm(proj, i_bias, f_bias, norm_w, state_nm, state_s, qsl, seq_lens, slot_table, H: int, D: int, Dv: int,
+          cap: float, eps: float):
+    """proj [T, 2*H*D + 2*H*Dv + 2*H] = [q | k | v | output gate | input gate | forget gate] (pre-activations);
+    state_nm fp32 [slots, H, Dn] (n in [:D], the running maximum at [D]); state_s fp32 [slots, H, D, Dv].
+        i = cap tanh((i_raw + i_bias) / cap), f = logsigmoid(cap tanh((f_raw + f_bias) / cap))
+        m' = max(f + m, i); S' = e^(f + m - m') S + e^(i - m') k v^T; n' likewise with k
+        o = S'^T q D^-1/2 / (max(|n' . q D^-1/2|, e^-m') + 1e-6)
+    out = o / rms(o) per head * norm_w * sigmoid(output gate)."""
+    T = proj.shape[0]
+    HD, HV = H * D, H * Dv
+    q = proj[:, :HD].float().view(T, H, D) * D ** -0.5
+    k = proj[:, HD: 2 * HD].float().view(T, H, D)
+    v = proj[:, 2 * HD: 2 * HD + HV].float().view(T, H, Dv)
+    og = proj[:, 2 * HD + HV: 2 * HD + 2 * HV].float()
+    ig = cap * torch.tanh((proj[:, 2 * HD + 2 * HV: 2 * HD + 2 * HV + H].float() + i_bias.float()) / cap)
+    fg = F.logsigmoid(cap * torch.tanh((proj[:, 2 * HD + 2 * HV + H:].float() + f_bias.float()) / cap))
+    out = torch.zeros((T, H, Dv), dtype=torch.float32, device=proj.device)
+    for s in range(seq_lens.shape[0]):
+        sl = int(seq_lens[s])
+        t0, t1 = int(qsl[s]), int(qsl[s + 1])
+        if sl <= 0 or t1 <= t0:
+            continue
+        slot = int(slot_table[s, 0])
+        if sl - (t1 - t0) > 0:
+            S, n, m = state_s[slot].clone(), state_nm[slot, :, :D].clone(), state_nm[slot, :, D].clone()
+        else:
+            S = torch.zeros((H, D, Dv), dtype=torch.float32, device=proj.device)
+            n, m = S.new_zeros((H, D)), S.new_zeros((H,))
+        for t in range(t0, t1):
+            m2 = torch.maximum(fg[t] + m, ig[t])
+            a, b = torch.exp(fg[t] + m - m2), torch.exp(ig[t] - m2)
+            S = a[:, None, None] * S + b[:, None, None] * k[t].unsqueeze(-1) * v[t].unsqueeze(1)
+            n = a[:, None] * n + b[:, None] * k[t]
+            m = m2
+            den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t]) / den[:, None]
+        state_s[slot] = S
+        state_nm[slot, :, :D] = n
+        state_nm[slot, :, D] = m
+    o = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+    o = o.view(T, HV) * norm_w.float() * torch.sigmoid(og)
+    return o.to(proj.dtype)
