@@ -143,7 +143,10 @@ def main() -> None:
                     help="instead of the flagship run: prefill / decode throughput of Nositar stacks beside a "
                          "sliding-window Llama and a Jamba stack of equal size (benchmarks/hybrid_compare.py; "
                          "--batch / --input-len / --output-len apply, one JSON line per model and size)")
-    ap.add_argument("--sizes", default="small,medium", help="--compare-nositar: small, medium, large")
+    ap.add_argument("--compare-rapovik", action="store_true",
+                    help="likewise for Rapovik stacks (latent window attention, Mamba-2, mLSTM, routed experts) beside "
+                         "a Jamba stack with routed experts of equal width, depth and feed-forward")
+    ap.add_argument("--sizes", default="small,medium", help="--compare-nositar / --compare-rapovik: small, medium, large")
     ap.add_argument("--rehearse-on-one-gpu", action="store_true", help="--disagg: every engine on GPU 0")
     ap.add_argument("--kv-push", action="store_true", help="--disagg: push blocks while prefilling (landing pool)")
     ap.add_argument("--num-prompts", type=int, default=200, help="--disagg: requests")
@@ -151,9 +154,9 @@ def main() -> None:
     a = ap.parse_args()
     if a.disagg:
         return run_disagg(a)
-    if a.compare_nositar:
+    if a.compare_nositar or a.compare_rapovik:
         from vllm_distributed_amd.benchmarks import hybrid_compare
-        argv = ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
+        argv = (["--models", "rapovik,jamba-moe"] if a.compare_rapovik else []) + ["--sizes", a.sizes, "--batch", str(32 if a.batch == 256 else a.batch),
                 "--input-len", str(2048 if a.input_len == 1024 else a.input_len),
                 "--output-len", str(64 if a.output_len == 128 else a.output_len)]
         hybrid_compare.main(argv + (["--enforce-eager"] if a.enforce_eager else []))

@@ -6,7 +6,9 @@ Weights are a dict of tensors under the checkpoint's names; ``cfg`` is the parse
 """
 from __future__ import annotations
 
+import json
 import math
+import os
 
 import torch
 
@@ -196,3 +198,117 @@ def forward(cfg, weights, tokens, dtype=torch.float32, want_layers=False):
         trail.append(x)
     logits = norm_around_zero(x, W["final.norm"], eps) @ W["head"].T
     return (logits, torch.stack(trail)) if want_layers else logits
+
+
+# ---- small random models ---------------------------------------------------------------------------------------------
+def attention_layer(heads=3, dim=12, rot_dim=8, vdim=20, kv_rank=24, window=9, base=100.0, rot_dims=None, scale=0.3,
+                    mlp="dense"):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": scale}
+    if window:
+        m["mask"] = {"size": window}
+    if base:
+        m["rot"] = {"base": base, "dims": rot_dims or rot_dim}
+    return {"type": "latent_attention", "mixer": m, "mlp": feed_forward(mlp)}
+
+
+def mamba_layer(heads=4, vdim=12, state=16, groups=2, conv=4, norm_groups=2, mlp="moe"):
+    return {"type": "mamba2", "mixer": {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv,
+                                        "norm_groups": norm_groups}, "mlp": feed_forward(mlp)}
+
+
+def mlstm_layer(heads=2, dim=12, vdim=20, gate_cap=15.0, mlp="dense"):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": gate_cap},
+            "mlp": feed_forward(mlp)}
+
+
+def feed_forward(kind, ff=40, limit=1.5, experts=6, top=2, groups=(3, 2), shared=24):
+    if kind is None or isinstance(kind, dict):
+        return kind
+    if kind == "dense":
+        return {"kind": "dense", "ff": ff, "limit": limit}
+    router = {"experts": experts, "top": top}
+    if groups:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    out = {"kind": "moe", "router": router, "expert": {"ff": ff // 2, "limit": limit}}
+    if shared:
+        out["shared"] = {"ff": shared, "limit": limit + 0.5}
+    return out
+
+
+def make_config(layers, vocab=96, width=48, eps=1e-5, loop=None):
+    cfg = {"architecture": "Rapovik", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": eps}}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+def make_weights(cfg, seed=0, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    Wd, V = cfg["width"], cfg["vocab"]
+
+    def rnd(*shape, s=1.0):
+        return torch.randn(*shape, generator=g) * s
+
+    def lin(o, i, s=1.0):
+        return rnd(o, i, s=s / math.sqrt(i))
+    W = {"embed": rnd(V, Wd), "head": lin(V, Wd, 2.0), "final.norm": rnd(Wd, s=0.1)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        for n in ("norm1", "norm1b"):
+            W[p + n] = rnd(Wd, s=0.1)
+        if L["type"] == "latent_attention":
+            H, D, P, E, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            W.update({p + "mix.q": lin(H * (D + P), Wd, 2.0), p + "mix.dkv": lin(R + P, Wd, 2.0),
+                      p + "mix.dkv.norm": 1.0 + rnd(R, s=0.1), p + "mix.uk": lin(H * D, R, 2.0),
+                      p + "mix.uv": lin(H * E, R), p + "mix.o": lin(Wd, H * E)})
+        elif L["type"] == "mamba2":
+            H, E, N, G, t = m["heads"], m["vdim"], m["state"], m["groups"], m["conv"]
+            inner, ch = H * E, H * E + 2 * G * N
+            W.update({p + "mix.in": lin(2 * inner + 2 * G * N + H, Wd, 1.5), p + "mix.conv": rnd(ch, t, s=0.5),
+                      p + "mix.conv.b": rnd(ch, s=0.2), p + "mix.dt_bias": rnd(H) - 1.0, p + "mix.A_log": rnd(H, s=0.5),
+                      p + "mix.D": 1.0 + rnd(H, s=0.2), p + "mix.norm": 1.0 + rnd(inner, s=0.1),
+                      p + "mix.o": lin(Wd, inner)})
+        else:
+            H, D, E = m["heads"], m["dim"], m["vdim"]
+            W.update({p + "mix.q": lin(H * D, Wd, 2.0), p + "mix.k": lin(H * D, Wd, 2.0), p + "mix.v": lin(H * E, Wd),
+                      p + "mix.g": lin(H * E, Wd), p + "mix.o": lin(Wd, H * E), p + "mix.norm": 1.0 + rnd(H * E, s=0.1),
+                      p + "mix.i": lin(H, Wd, 2.0), p + "mix.i.b": rnd(H), p + "mix.f": lin(H, Wd, 2.0),
+                      p + "mix.f.b": rnd(H) + 3.0})
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        for n in ("norm2", "norm2b"):
+            W[p + n] = rnd(Wd, s=0.1)
+        if mlp.get("kind", "dense") == "dense":
+            ff = mlp["ff"]
+            W.update({p + "mlp.gate": lin(ff, Wd, 2.5), p + "mlp.gate.b": rnd(ff, s=0.3), p + "mlp.up": lin(ff, Wd, 2.5),
+                      p + "mlp.up.b": rnd(ff, s=0.3), p + "mlp.down": lin(Wd, ff), p + "mlp.down.b": rnd(Wd, s=0.1)})
+        else:
+            E_, ff = mlp["router"]["experts"], mlp["expert"]["ff"]
+            W[p + "mlp.router"] = lin(E_, Wd, 3.0)
+            W[p + "mlp.correction"] = rnd(E_, s=0.3) - 0.5         # choice scores of either sign
+            for e in range(E_):
+                W.update({f"{p}mlp.e{e}.gate": lin(ff, Wd, 2.5), f"{p}mlp.e{e}.up": lin(ff, Wd, 2.5),
+                          f"{p}mlp.e{e}.down": lin(Wd, ff)})
+            if mlp.get("shared"):
+                fs = mlp["shared"]["ff"]
+                W.update({p + "mlp.shared.gate": lin(fs, Wd, 2.5), p + "mlp.shared.up": lin(fs, Wd, 2.5),
+                          p + "mlp.shared.down": lin(Wd, fs)})
+    # the checkpoint holds bfloat16: round once, so that oracle and engine read the same numbers
+    return {k: v.to(dtype) for k, v in W.items()}
+
+
+def save_checkpoint(folder, cfg, W):
+    from safetensors.torch import save_file
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in W.items()}, os.path.join(folder, "model.safetensors"))
+    return folder
+
+
+def logit_error(got, want):
+    """Root mean square difference over the vocabulary with the mean taken off, relative to the logits' own spread."""
+    d = torch.as_tensor(got).float() - torch.as_tensor(want).float()
+    d = d - d.mean(-1, keepdim=True)
+    return (d.pow(2).mean(-1).sqrt() / torch.as_tensor(want).float().std(-1).clamp_min(1e-6)).max().item()

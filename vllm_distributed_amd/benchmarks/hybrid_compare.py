@@ -1,6 +1,8 @@
-"""Prefill and decode throughput of a Nositar stack beside the closest existing models of equal size, random weights.
+"""Prefill and decode throughput of a Nositar or Rapovik stack beside the closest existing models of equal size, random
+weights.
 
     python bench.py --compare-nositar [--sizes small,medium] [--batch 32] [--input-len 2048] [--output-len 64]
+    python bench.py --compare-rapovik [...]        (rapovik beside jamba-moe)
 
 Per size three engines run one after the other, each in a process of its own (``--one`` is the child's entry):
   nositar      alternating sigmoid head-mixing attention (window + kept first tokens) and gated delta-rule layers,
@@ -8,6 +10,9 @@ Per size three engines run one after the other, each in a process of its own (``
   llama-swa    a Llama stack of the same width, depth, heads and feed-forward with the same sliding window (the
                framework's softmax attention kernels)
   jamba        the framework's attention + recurrent (Mamba) hybrid of the same width, depth and feed-forward
+  jamba-moe    the same with 8 routed experts (two per token) in every other layer
+  rapovik      latent window attention, Mamba-2 and mLSTM mixers in turn over an fp32 residual with norms around every
+               sub-layer; clamped gated feed-forwards, dense and routed (8 experts, two per token, one shared) in turn
 Prefill: ``batch`` prompts of ``input-len`` tokens, one generated token.  Decode: the same requests generating
 ``output-len`` tokens, the prefill time taken off.  One JSON line per (size, model).
 """
@@ -61,7 +66,34 @@ def jamba_config(s: dict) -> dict:
             "torch_dtype": "bfloat16"}
 
 
-MODELS = {"nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config}
+def jamba_moe_config(s: dict) -> dict:
+    """Jamba with routed experts (8, two per token) in every other layer, as the checkpoints of that family have."""
+    return dict(jamba_config(s), num_experts=8, num_experts_per_tok=2)
+
+
+def rapovik_config(s: dict) -> dict:
+    """Per four layers: latent window attention, Mamba-2, mLSTM, Mamba-2; dense feed-forwards alternate with routed
+    experts (8, two per token from the better of two groups, plus a shared expert of a quarter of the width)."""
+    w, ff = s["width"], s["ff"]
+    rank, rot = (128, 32) if w <= 1024 else (512, 64)
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    moe = {"kind": "moe", "router": {"experts": 8, "top": 2, "groups": {"count": 2, "keep": 1}},
+           "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": ff // 4, "limit": 7.0}}
+    att = {"type": "latent_attention",
+           "mixer": {"heads": s["heads"], "dim": s["dim"], "rot_dim": rot, "vdim": s["dim"], "kv_rank": rank,
+                     "scale": (s["dim"] + rot) ** -0.5, "mask": {"size": s["window"]},
+                     "rot": {"base": 10000.0, "dims": rot}}}
+    mamba = {"type": "mamba2", "mixer": {"heads": 2 * w // 64, "vdim": 64, "state": 64, "groups": 1, "conv": 4,
+                                         "norm_groups": 1}}
+    mh = max(w // 128, 1)
+    mlstm = {"type": "mlstm", "mixer": {"heads": mh, "dim": 64, "vdim": 2 * w // mh, "gate_cap": 15.0}}
+    cycle = [att, mamba, mlstm, mamba]
+    return {"architecture": "Rapovik", "vocab": s["vocab"], "width": w, "norm": {"eps": 1e-6},
+            "layers": [dict(cycle[i % 4], mlp=dense if i % 2 == 0 else moe) for i in range(s["layers"])]}
+
+
+MODELS = {"nositar": nositar_config, "llama-swa": llama_config, "jamba": jamba_config, "jamba-moe": jamba_moe_config,
+          "rapovik": rapovik_config}
 
 
 def run_one(kind: str, size: str, batch: int, input_len: int, output_len: int, eager: bool) -> dict:

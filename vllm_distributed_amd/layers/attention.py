@@ -464,10 +464,8 @@ class MLAAttention(nn.Module):
         # request (a full-attention layer to the cache manager); the kernel never loads them.
         self.sliding_window = int(sliding_window or 0)
         # False: the cache keeps the latent rows only and ``forward_cached`` attends over them with the kernel for
-        # any sizes and windows (ops.latent_window_attention); the caller writes the rows itself
+        # any sizes and types (ops.latent_window_attention) instead of the MFMA kernel, which wants the copy
         self.transposed_copy = bool(transposed_copy)
-        if self.sliding_window and self.transposed_copy:
-            raise ValueError("windowed latent attention runs on the rows-only cache (transposed_copy=False)")
         self.dk, self.dv = kv_lora_rank + rope_dim, kv_lora_rank
         self.scale = float(scale)
         self.layer_name = prefix
@@ -510,14 +508,26 @@ class MLAAttention(nn.Module):
         return out
 
     def forward_cached(self, q: torch.Tensor) -> torch.Tensor:
-        """Attention over rows the caller has already written to ``k_cache`` for this step's tokens (rows-only
-        cache).  q [T, H, dk]; returns [T, H, kv_lora_rank]."""
+        """Attention over rows the caller has already written to the cache for this step's tokens.
+        q [T, H, dk]; returns [T, H, kv_lora_rank]."""
         md: Optional[AttentionMetadata] = get_forward_context().attn_metadata
         T = q.shape[0]
         if md is None or self.k_cache is None:
             return torch.zeros((T, self.num_heads, self.dv), dtype=q.dtype, device=q.device)
         n = md.num_actual_tokens
         S = md.num_decode_seqs + md.num_prefill_seqs
+        if self.transposed_copy:
+            out = torch.empty((T, self.num_heads, self.dv), dtype=q.dtype, device=q.device)
+            if n < T:
+                out[n:].zero_()
+            nsplit = 1
+            if md.max_query_len <= 4:           # few query tokens: split the keys so that the launch fills the chip
+                keys = min(self.max_model_len, self.sliding_window + 32) if self.sliding_window else self.max_model_len
+                nsplit = ops.decode_num_splits(S * max(self.num_heads // 16, 1), 1, keys)
+            ops.mla_attention(out[:n], q[:n], self.k_cache, self.v_cache, md.block_table[:S], md.seq_lens[:S],
+                              md.query_start_loc[:S + 1], self.scale, md.max_query_len, nsplit, self._kv_scale_float,
+                              window=self.sliding_window)
+            return out
         out = ops.latent_window_attention(q[:n], self.k_cache, md.block_table[:S], md.seq_lens[:S],
                                           md.query_start_loc[:S + 1], self.scale, self.sliding_window, self.dv,
                                           md.max_query_len)

@@ -11,7 +11,7 @@ The rotation turns the pairs (2i, 2i + 1), i < rot_dims / 2, of the P rotated va
 (angles, cosines and sines in fp32; values past rot_dims pass unchanged).  The key up-projection is folded into the
 query (q_abs = W_uk_h^T q_plain, so the score is q_abs . c + q_rot . k_rot) and the value up-projection is applied
 after the attention, which then runs over the cached rows [c | k_rot] for all heads alike: the cache holds R + P
-values per token (``MLAAttention`` with the rows-only cache).  A mixer whose weights serve several passes of a looped
+values per token (``MLAAttention``; the MFMA kernel keeps a transposed copy of c beside them).  A mixer whose weights serve several passes of a looped
 stack owns one cache per pass.
 Kernels: ops/csrc/latent_attention.hip.
 """
@@ -22,7 +22,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
-from .. import ops
+from .. import envs, ops
 from ..config import get_current_vllm_config
 from ..forward_context import get_forward_context
 from ..parallel.state import get_tensor_model_parallel_world_size
@@ -70,10 +70,15 @@ class WindowedLatentAttention(nn.Module):
         self.o_proj = RowParallelLinear(H * Dv, hidden_size, bias=False, quant_config=quant_config,
                                         prefix=f"{prefix}.o_proj")
         self.c_norm = _fp32_param((R,))
+        cfg = get_current_vllm_config()
+        # 16-bit activations and sizes the MFMA kernel is built for: that kernel (it wants a transposed copy of the
+        # latent beside the rows); anything else, fp32 included: the kernel for any sizes on the rows alone
+        self.use_mfma = bool(cfg.device_config.device != "cpu" and not envs.VDA_FORCE_TORCH_OPS and envs.VDA_MLA
+                             and cfg.model_config.dtype in (torch.bfloat16, torch.float16)
+                             and cfg.cache_config.cache_dtype == "auto" and (R + P, R) in ops.MLA_KERNEL_SIZES)
         self.attn = nn.ModuleList([
             MLAAttention(H, R, P, float(scale), prefix=f"{prefix}.attn.{i}", sliding_window=int(window or 0),
-                         transposed_copy=False) for i in range(passes)])
-        cfg = get_current_vllm_config()
+                         transposed_copy=self.use_mfma) for i in range(passes)])
         self.max_len = int(cfg.model_config.max_model_len) + 1
         self.rot_base = float(rot_base) if rot_base else 0.0
         self._cos_sin: Optional[torch.Tensor] = None
@@ -113,7 +118,8 @@ class WindowedLatentAttention(nn.Module):
             if n < T:
                 qf[n:, :, R:].zero_()
             ops.latent_norm_rope_cache(q[:n], down[:n], self.c_norm, self._tables(q.device), positions[:n], qf[:n],
-                                       attn.k_cache, md.slot_mapping[:n], H, D, P, R, self.rot_dims, self.eps)
+                                       attn.k_cache, md.slot_mapping[:n], H, D, P, R, self.rot_dims, self.eps,
+                                       attn.v_cache if self.use_mfma else None)
             o_lat = attn.forward_cached(qf)
         o = torch.bmm(o_lat.transpose(0, 1), w_uv_t).transpose(0, 1)
         return self.o_proj(o.reshape(T, H * Dv))

@@ -334,11 +334,14 @@ def merge_attn_states(prefix, prefix_lse, suffix, suffix_lse, return_lse: bool =
 
 
 # ---- multi-head latent attention ------------------------------------------------------------
+MLA_KERNEL_SIZES = ((576, 512), (96, 64), (160, 128))       # (row width, latent width) the MFMA kernel is built for
+
+
 def mla_supported(dk: int, dv: int, dtype: torch.dtype, on_device: bool) -> bool:
     """Latent sizes the MLA kernel is built for (DeepSeek-V2/V3: 576 / 512, plus two small ones)."""
     if not on_device or envs.VDA_FORCE_TORCH_OPS:
         return True
-    return dtype in (torch.bfloat16, torch.float16) and (dk, dv) in ((576, 512), (96, 64), (160, 128))
+    return dtype in (torch.bfloat16, torch.float16) and (dk, dv) in MLA_KERNEL_SIZES
 
 
 def mla_cache_write(kv_c: torch.Tensor, k_pe: torch.Tensor, kc: torch.Tensor, vt: torch.Tensor,
@@ -357,13 +360,13 @@ def mla_cache_write(kv_c: torch.Tensor, k_pe: torch.Tensor, kc: torch.Tensor, vt
 
 def mla_attention(out: torch.Tensor, q: torch.Tensor, kc: torch.Tensor, vt: torch.Tensor, block_table: torch.Tensor,
                   seq_lens: torch.Tensor, q_start_loc: torch.Tensor, scale: float, max_query_len: int,
-                  num_splits: int = 1, kv_scale: float = 1.0) -> torch.Tensor:
+                  num_splits: int = 1, kv_scale: float = 1.0, window: int = 0) -> torch.Tensor:
     """Causal multi-query attention of q [T, H, DK] over the latent cache; out [T, H, DV] stays in latent
     space (the caller applies the value up-projection).  Decode and (chunked) prefill are one path."""
     T, H, DK = q.shape
     DV = vt.shape[1]
     if not _dev(q):
-        out.copy_(R.mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale))
+        out.copy_(R.mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale, window))
         return out
     part_out = part_lse = None
     if num_splits > 1:
@@ -373,7 +376,8 @@ def mla_attention(out: torch.Tensor, q: torch.Tensor, kc: torch.Tensor, vt: torc
     N.call("vda_mla_attention", out.data_ptr(), q.data_ptr(), kc.data_ptr(), vt.data_ptr(), block_table.data_ptr(),
            seq_lens.data_ptr(), q_start_loc.data_ptr(), N.ptr(part_out), N.ptr(part_lse), seq_lens.shape[0], T, H, DK,
            DV, kc.shape[1], block_table.stride(0), num_splits, max(int(max_query_len), 1), q.stride(0),
-           out.stride(0), scale, N.dt(q.dtype), int(kc.dtype == torch.float8_e4m3fn), float(kv_scale), N.stream())
+           out.stride(0), scale, N.dt(q.dtype), int(kc.dtype == torch.float8_e4m3fn), float(kv_scale), int(window),
+           N.stream())
     return out
 
 
@@ -1098,6 +1102,26 @@ def moe_rows_form(num_pairs: int, num_experts: int, rows: int, weight_bytes: int
     return wide if avg >= 8 and (fills or avg >= 64) else 0
 
 
+def moe_pairs_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> bool:
+    """The plain-arithmetic expert kernel: any widths, weights of the activations' type (16-bit or fp32)."""
+    return (x.dtype in (torch.bfloat16, torch.float16, torch.float32) and w13.dtype == x.dtype and w2.dtype == x.dtype
+            and (w13.shape[2] + w13.shape[1] // 2) * 4 <= 60 * 1024 and w13.is_contiguous() and w2.is_contiguous())
+
+
+def _moe_pairs(x, w13, w2, topk_w, topk_ids, activation: str, act_limit: float):
+    """Experts of sizes the MFMA kernels are not built for: one workgroup per (token, choice) pair
+    (ops/csrc/moe.hip, vda_moe_pairs); sums over a token's choices in a fixed order."""
+    T, H = x.shape
+    k = topk_ids.shape[1]
+    I, Ho = w13.shape[1] // 2, w2.shape[1]
+    out = torch.empty((T, Ho), dtype=x.dtype, device=x.device)
+    part = torch.empty((T * k, Ho), dtype=torch.float32, device=x.device)
+    N.call("vda_moe_pairs", out.data_ptr(), out.stride(0), part.data_ptr(), x.data_ptr(), x.stride(0), w13.data_ptr(),
+           w2.data_ptr(), topk_w.contiguous().data_ptr(), topk_ids.contiguous().data_ptr(), T, H, I, Ho, k,
+           N.ACT[activation], float(act_limit), N.dt(x.dtype), N.stream())
+    return out
+
+
 MOE_ACTIVATIONS = ("silu", "gelu", "gelu_tanh", "gelu_pytorch_tanh", "relu", "relu2", "clamped_swiglu")
 
 
@@ -1123,6 +1147,9 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
     if _dev(x) and block_scales and not moe_tiled_ok(x, w13, w2):
         raise RuntimeError(f"block-scaled expert shapes {tuple(w13.shape)} / {tuple(w2.shape)} are outside the tiled "
                            "fp8 GEMM (hidden and expert width must be multiples of 128)")
+    if _dev(x) and not moe_grouped_ok(x, w13, w2) and not moe_tiled_ok(x, w13, w2) and moe_pairs_ok(x, w13, w2) \
+            and w13_scale is None and w2_scale is None:
+        return _moe_pairs(_contig_last(x), w13, w2, topk_w, topk_ids, activation, act_limit)
     if not _dev(x) or (not moe_grouped_ok(x, w13, w2) and not moe_tiled_ok(x, w13, w2)):
         if _dev(x) and torch.cuda.is_current_stream_capturing():
             raise RuntimeError(
@@ -1421,14 +1448,15 @@ def residual_norms(x: torch.Tensor, y: Optional[torch.Tensor] = None, w_post: Op
 def latent_norm_rope_cache(q: torch.Tensor, down: torch.Tensor, c_weight: torch.Tensor, cos_sin: torch.Tensor,
                            positions: torch.Tensor, qf: torch.Tensor, kc: Optional[torch.Tensor],
                            slot_mapping: torch.Tensor, H: int, D: int, P: int, rank: int, rot_dims: int,
-                           eps: float) -> None:
+                           eps: float, vt: Optional[torch.Tensor] = None) -> None:
     """Per token: the cache row [down[:rank] / rms * c_weight | down[rank:] with its first ``rot_dims`` values rotated] goes
     to ``kc`` [blocks, bs, rank + P] at ``slot_mapping``; the last P values of every query head (q [T, H * (D + P)]),
     rotated alike, go to qf[:, h, rank:] (qf [T, H, rank + P]).  Pairs (2i, 2i + 1) turn by the angle whose cosine and sine
-    are cos_sin[position, i] and cos_sin[position, rot_dims / 2 + i] (fp32)."""
+    are cos_sin[position, i] and cos_sin[position, rot_dims / 2 + i] (fp32).  ``vt`` [blocks, rank, bs]: a transposed
+    copy of the rows' first ``rank`` values, for the kernel that wants one."""
     if not _dev(q):
         return R.latent_norm_rope_cache(q, down, c_weight, cos_sin, positions, qf, kc, slot_mapping, H, D, P, rank,
-                                        rot_dims, eps)
+                                        rot_dims, eps, vt)
     T = q.shape[0]
     assert q.stride(1) == 1 and down.stride(1) == 1 and qf.is_contiguous() and kc.is_contiguous()
     assert q.dtype == down.dtype == qf.dtype == kc.dtype and kc.shape[2] == rank + P and qf.shape == (T, H, rank + P)
@@ -1436,7 +1464,7 @@ def latent_norm_rope_cache(q: torch.Tensor, down: torch.Tensor, c_weight: torch.
     assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int64 and c_weight.dtype == torch.float32
     N.call("vda_latent_norm_rope_cache", q.data_ptr(), q.stride(0), down.data_ptr(), down.stride(0),
            c_weight.data_ptr(), cos_sin.data_ptr(), positions.data_ptr(), qf.data_ptr(), kc.data_ptr(),
-           slot_mapping.data_ptr(), T, H, D, P, rank, rot_dims, kc.shape[1], float(eps), N.dt(q.dtype), N.stream())
+           vt.data_ptr() if vt is not None and vt.numel() else None, slot_mapping.data_ptr(), T, H, D, P, rank, rot_dims, kc.shape[1], float(eps), N.dt(q.dtype), N.stream())
 
 
 def latent_window_attention(q: torch.Tensor, kc: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor,

@@ -7,7 +7,8 @@
 //
 //   vda_latent_norm_rope_cache   per token: c = down[:R] / rms * weight, rotate down[R:] and every query head's last
 //                                P values (interleaved pairs, angles from an fp32 cos | sin table), write the cache
-//                                row and qf[:, :, R:] in one launch
+//                                row (and, for the MFMA kernel of mla.hip, the transposed copy of c) and
+//                                qf[:, :, R:] in one launch
 //   vda_latent_window_attention  softmax(scale * qf . row) over the keys j <= i, i - j < window; scores, softmax and
 //                                the weighted sum in fp32.  One workgroup per (sequence, tile of query tokens) walks
 //                                the visible keys in tiles through LDS with a running maximum and sum per row; keys
@@ -19,8 +20,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_norm_rope_cache_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ down, long down_stride,
     const float* __restrict__ c_weight, const float* __restrict__ cos_sin, const long* __restrict__ positions,
-    T* __restrict__ qf, T* __restrict__ kc, const long* __restrict__ slot_mapping, int H, int D, int P, int R,
-    int rot, int bs, float eps) {
+    T* __restrict__ qf, T* __restrict__ kc, T* __restrict__ vt, const long* __restrict__ slot_mapping, int H, int D,
+    int P, int R, int rot, int bs, float eps) {
   __shared__ float red[16];
   const long t = blockIdx.x;
   const int tid = threadIdx.x;
@@ -37,7 +38,12 @@ __global__ __launch_bounds__(256) void latent_norm_rope_cache_kernel(
   const long slot = slot_mapping[t];
   T* row = slot >= 0 ? kc + slot * (long)DK : nullptr;      // slot = block * bs + offset, rows are contiguous
   if (row) {
-    for (int c = tid; c < R; c += 256) row[c] = (T)((float)dr[c] * rs * c_weight[c]);
+    T* col = vt ? vt + ((slot / bs) * R) * (long)bs + slot % bs : nullptr;     // vt [blocks, R, bs]
+    for (int c = tid; c < R; c += 256) {
+      const T v = (T)((float)dr[c] * rs * c_weight[c]);
+      row[c] = v;
+      if (col) col[(long)c * bs] = v;
+    }
     for (int i = tid; i < P; i += 256) {
       float v;
       if (i < rot) {
@@ -70,13 +76,13 @@ __global__ __launch_bounds__(256) void latent_norm_rope_cache_kernel(
 
 VDA_EXPORT int vda_latent_norm_rope_cache(const void* q, long q_stride, const void* down, long down_stride,
                                           const float* c_weight, const float* cos_sin, const long* positions,
-                                          void* qf, void* kc, const long* slot_mapping, int T, int H, int D, int P,
-                                          int R, int rot, int bs, float eps, int dtype, hipStream_t st) {
+                                          void* qf, void* kc, void* vt, const long* slot_mapping, int T, int H, int D,
+                                          int P, int R, int rot, int bs, float eps, int dtype, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > P || (rot & 1)) return -1;
 #define L(TT) hipLaunchKernelGGL((latent_norm_rope_cache_kernel<TT>), dim3(T), dim3(256), 0, st, (const TT*)q,      \
                                  q_stride, (const TT*)down, down_stride, c_weight, cos_sin, positions, (TT*)qf,      \
-                                 (TT*)kc, slot_mapping, H, D, P, R, rot, bs, eps)
+                                 (TT*)kc, (TT*)vt, slot_mapping, H, D, P, R, rot, bs, eps)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
@@ -90,8 +96,11 @@ VDA_EXPORT int vda_latent_norm_rope_cache(const void* q, long q_stride, const vo
 template <typename T, int NACC>
 __global__ __launch_bounds__(256) void latent_window_attention_kernel(
     T* __restrict__ out, const T* __restrict__ qf, const T* __restrict__ kc, const int* __restrict__ block_table,
-    long bt_stride, const int* __restrict__ seq_lens, const int* __restrict__ qsl, float scale, int window, int H,
-    int DK, int R, int bs, int BQ, int BK) {
+    long bt_stride, const int* __restrict__ seq_lens, const int* __restrict__ qsl, float scale, int window, int HT,
+    int HG, int DK, int R, int bs, int BQ, int BK) {
+  // HT heads in all; this workgroup takes the H heads from h0 on (grid.z deals groups of HG heads)
+  const int h0 = blockIdx.z * HG;
+  const int H = min(HG, HT - h0);
   extern __shared__ float lds[];
   const int Dq = (DK + 3) / 4 * 4 + 1;          // padded row of q and the latent rows (odd: no bank conflicts
   const int RS = BK + 1;                        //  when lanes walk rows)
@@ -115,7 +124,7 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(
 
   for (int e = tid; e < M * DK; e += 256) {
     const int d = e % DK, m = e / DK;             // m = i * H + h
-    qs[m * Dq + d] = (m / H) < nq ? (float)qf[((long)(t0 + i0) * H + m) * DK + d] * scale : 0.f;
+    qs[m * Dq + d] = (m / H) < nq ? (float)qf[((long)(t0 + i0 + m / H) * HT + h0 + m % H) * DK + d] * scale : 0.f;
   }
   for (int m = tid; m < M; m += 256) { rm[m] = -INFINITY; rl[m] = 0.f; }
   float acc[NACC];
@@ -190,7 +199,7 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(
       const int d = e % R, m = e / R;
       if (m / H < nq) {
         const float l = rl[m];
-        out[((long)(t0 + i0) * H + m) * R + d] = (T)(l > 0.f ? acc[n] / l : 0.f);
+        out[((long)(t0 + i0 + m / H) * HT + h0 + m % H) * R + d] = (T)(l > 0.f ? acc[n] / l : 0.f);
       }
     }
   }
@@ -203,23 +212,27 @@ VDA_EXPORT int vda_latent_window_attention(void* out, const void* qf, const void
   if (S <= 0 || max_q <= 0) return 0;
   if (H <= 0 || R <= 0 || R > DK) return -1;
   // tile sizes: the largest query tile (then key tile) whose accumulators fit 64 registers per thread, whose rows
-  // fit one workgroup and whose tiles fit 96 KiB of LDS; single decoded tokens take a one-token tile
+  // fit one workgroup and whose tiles fit 96 KiB of LDS; single decoded tokens take a one-token tile; heads are
+  // dealt to several workgroups when one token's heads alone are too many for that
   const int Dq = (DK + 3) / 4 * 4 + 1;
-  auto lds_of = [&](int bq, int bk) {
-    return ((size_t)bq * H * Dq + (size_t)bk * Dq + (size_t)bq * H * (bk + 1) + 3 * (size_t)bq * H) * 4;
+  auto lds_of = [&](int bq, int bk, int hg) {
+    return ((size_t)bq * hg * Dq + (size_t)bk * Dq + (size_t)bq * hg * (bk + 1) + 3 * (size_t)bq * hg) * 4;
   };
-  int BQ = 0, BK = 0;
-  for (int bq = 16; bq >= 1 && !BQ; bq >>= 1) {
-    if (bq > 1 && bq / 2 >= max_q) continue;
-    if ((size_t)bq * H * R > 256 * 64 || bq * H > 256) continue;
-    for (int bk = 64; bk >= 1; bk >>= 1)
-      if (lds_of(bq, bk) <= 96 * 1024) { BQ = bq; BK = bk; break; }
+  int BQ = 0, BK = 0, HG = H;
+  for (; HG >= 1 && !BQ; HG = HG > 1 ? (HG + 1) / 2 : 0) {
+    for (int bq = 16; bq >= 1 && !BQ; bq >>= 1) {
+      if (bq > 1 && bq / 2 >= max_q) continue;
+      if ((size_t)bq * HG * R > 256 * 64 || bq * HG > 256) continue;
+      for (int bk = 64; bk >= 8; bk >>= 1)
+        if (lds_of(bq, bk, HG) <= 96 * 1024) { BQ = bq; BK = bk; break; }
+    }
+    if (BQ) break;
   }
   if (!BQ) return -2;
-  const size_t lds = lds_of(BQ, BK);
-  const int per = (BQ * H * R + 255) / 256;
+  const size_t lds = lds_of(BQ, BK, HG);
+  const int per = (BQ * HG * R + 255) / 256;
   const int NACC = per <= 8 ? 8 : per <= 16 ? 16 : per <= 32 ? 32 : 64;
-  dim3 grid((max_q + BQ - 1) / BQ, S), block(256);
+  dim3 grid((max_q + BQ - 1) / BQ, S, (H + HG - 1) / HG), block(256);
 #define L2(TT, NA)                                                                                                  \
   do {                                                                                                              \
     if (lds > 48 * 1024) {                                                                                          \
@@ -228,7 +241,8 @@ VDA_EXPORT int vda_latent_window_attention(void* out, const void* qf, const void
       if (e != hipSuccess) return (int)e;                                                                           \
     }                                                                                                               \
     hipLaunchKernelGGL((latent_window_attention_kernel<TT, NA>), grid, block, lds, st, (TT*)out, (const TT*)qf,     \
-                       (const TT*)kc, block_table, bt_stride, seq_lens, qsl, scale, window, H, DK, R, bs, BQ, BK);  \
+                       (const TT*)kc, block_table, bt_stride, seq_lens, qsl, scale, window, H, HG, DK, R, bs, BQ,   \
+                       BK);                                                                                         \
   } while (0)
 #define L(TT)                                                                                                       \
   do {                                                                                                              \

@@ -84,6 +84,7 @@ struct MlaParams {
   long q_stride, out_stride;
   float scale;              // softmax scale, times the cache scale for an fp8 cache
   float v_scale;            // 1, or the cache scale for an fp8 cache
+  int window;               // > 0: a query at position i sees the keys j with 0 <= i - j < window
 };
 
 template <typename T, int DK, int DV, bool F8>
@@ -120,13 +121,19 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = valid ? ld16<V8>(qp + 8 * s) : V8{};
   }
-  int hi = limit;
+  const int first = p.window > 0 ? max(limit - p.window, 0) : 0;      // first visible key of this column
+  int hi = limit, lo = valid ? first : 0x7fffffff;
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) hi = max(hi, __shfl_xor(hi, o, 64));
-  // key steps of 32: partition over grid.z, then deal to the 4 waves
+  for (int o = 32; o > 0; o >>= 1) {
+    hi = max(hi, __shfl_xor(hi, o, 64));
+    lo = min(lo, __shfl_xor(lo, o, 64));
+  }
+  // key steps of 32 (those before every column's window are never loaded): partition over grid.z, then deal to
+  // the 4 waves
   int step_hi = (hi + 31) / 32;
-  const int per = (step_hi + p.nsplit - 1) / p.nsplit;
-  const int a0 = blockIdx.z * per;
+  const int step_lo = min(lo / 32, step_hi);
+  const int per = (step_hi - step_lo + p.nsplit - 1) / p.nsplit;
+  const int a0 = step_lo + blockIdx.z * per;
   step_hi = min(step_hi, a0 + per);
 
   float m = -INFINITY, l = 0.f;
@@ -155,7 +162,7 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
     float mx = -INFINITY;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      sv[j] = (tb + j < limit) ? sv[j] * sc : -INFINITY;
+      sv[j] = (tb + j < limit && tb + j >= first) ? sv[j] * sc : -INFINITY;
       mx = fmaxf(mx, sv[j]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -297,7 +304,7 @@ VDA_EXPORT int vda_mla_attention(void* out, const void* q, const void* kc, const
                                  const int* seq_lens, const int* q_start_loc, float* part_out, float* part_lse,
                                  int S, int T_tokens, int H, int DK, int DV, int BS, int max_blocks, int nsplit,
                                  int max_q, long q_stride, long out_stride, float scale, int dtype, int kv_fp8,
-                                 float kv_scale, hipStream_t st) {
+                                 float kv_scale, int window, hipStream_t st) {
   if (S <= 0 || T_tokens <= 0) return 0;
   if (!vda_mla_supported(DK, DV) || BS % 8 || nsplit < 1 || nsplit > 64 || (nsplit > 1 && (!part_out || !part_lse)))
     return -1;      // (the reduce kernel keeps one partition per lane)
@@ -307,6 +314,7 @@ VDA_EXPORT int vda_mla_attention(void* out, const void* q, const void* kc, const
   p.H = H; p.BS = BS; p.max_blocks = max_blocks; p.nsplit = nsplit;
   p.q_stride = q_stride; p.out_stride = out_stride;
   p.scale = scale * (kv_fp8 ? kv_scale : 1.f); p.v_scale = kv_fp8 ? kv_scale : 1.f;
+  p.window = window > 0 ? window : 0;
   const bool f8 = kv_fp8 != 0;
 #define BYD(TT) do { if (DK == 576) launch_mla<TT, 576, 512>(p, S, T_tokens, max_q, f8, st);      \
                      else if (DK == 96) launch_mla<TT, 96, 64>(p, S, T_tokens, max_q, f8, st);    \

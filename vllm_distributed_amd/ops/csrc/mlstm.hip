@@ -15,7 +15,7 @@
 // by one from the carried state, so results do not depend on how a prompt is cut.
 #include "common.h"
 
-#define MLSTM_TCH 16
+#define MLSTM_TCH_MAX 16          // tokens staged through LDS at a time (fewer for very wide heads)
 
 __device__ __forceinline__ float logsigmoid_f(float x) {
   // -softplus(-x), stable for both signs
@@ -27,15 +27,15 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
     float* __restrict__ o_raw, const T* __restrict__ proj, long p_stride, const float* __restrict__ i_bias,
     const float* __restrict__ f_bias, float* __restrict__ state_nm, float* __restrict__ state_s,
     const int* __restrict__ qsl, const int* __restrict__ seq_lens, const int* __restrict__ slot_table,
-    long st_stride, int H, int D, int Dv, int Dn, int LPC, float cap) {
+    long st_stride, int H, int D, int Dv, int Dn, int LPC, int TCH, float cap) {
   extern __shared__ float lds[];
   const int DP = LPC * DPT;                       // D rounded up; the tail stays zero
   const int CW = 256 / LPC;                       // value columns of this workgroup
   float* qs = lds;                                // [TCH][DP]
-  float* ks = qs + MLSTM_TCH * DP;                // [TCH][DP]
-  float* vs = ks + MLSTM_TCH * DP;                // [TCH][CW]
-  float* gi = vs + MLSTM_TCH * CW;                // [TCH]
-  float* gf = gi + MLSTM_TCH;                     // [TCH]
+  float* ks = qs + TCH * DP;                      // [TCH][DP]
+  float* vs = ks + TCH * DP;                      // [TCH][CW]
+  float* gi = vs + TCH * CW;                      // [TCH]
+  float* gf = gi + TCH;                           // [TCH]
 
   const int s = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
   const int sl = seq_lens[s];
@@ -68,10 +68,10 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
   const T* pf = pi + H;
   const float bi = i_bias[h], bf = f_bias[h];
 
-  for (int c0 = 0; c0 < L; c0 += MLSTM_TCH) {
-    const int nt = min(MLSTM_TCH, L - c0);
+  for (int c0 = 0; c0 < L; c0 += TCH) {
+    const int nt = min(TCH, L - c0);
     __syncthreads();
-    for (int e = tid; e < MLSTM_TCH * DP; e += 256) {
+    for (int e = tid; e < TCH * DP; e += 256) {
       const int d = e % DP, tt = e / DP;
       float qv = 0.f, kv = 0.f;
       if (tt < nt && d < D) {
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(
       qs[e] = qv;
       ks[e] = kv;
     }
-    for (int e = tid; e < MLSTM_TCH * CW; e += 256) {
+    for (int e = tid; e < TCH * CW; e += 256) {
       const int c = e % CW, tt = e / CW;
       vs[e] = (tt < nt && blockIdx.x * CW + c < Dv) ? (float)pv[(long)(t0 + c0 + tt) * p_stride + c] : 0.f;
     }
@@ -161,7 +161,10 @@ VDA_EXPORT int vda_mlstm(void* out, long o_stride, float* o_raw, const void* pro
   if (per > 32) return -2;                       // D beyond 2048
   const int DPT = per <= 8 ? 8 : per <= 16 ? 16 : 32;
   const int CW = 256 / LPC;
-  const size_t lds = ((size_t)2 * MLSTM_TCH * LPC * DPT + (size_t)MLSTM_TCH * CW + 2 * MLSTM_TCH) * 4;
+  int TCH = MLSTM_TCH_MAX;
+  auto lds_of = [&](int tch) { return ((size_t)2 * tch * LPC * DPT + (size_t)tch * CW + 2 * tch) * 4; };
+  while (TCH > 1 && lds_of(TCH) > 60 * 1024) TCH >>= 1;
+  const size_t lds = lds_of(TCH);
   dim3 grid((Dv + CW - 1) / CW, H, S), block(256);
   const long gate_off = 2L * H * D + (long)H * Dv;
 #define L2(TT, DD)                                                                                                   \
@@ -172,7 +175,7 @@ VDA_EXPORT int vda_mlstm(void* out, long o_stride, float* o_raw, const void* pro
       if (e != hipSuccess) return (int)e;                                                                            \
     }                                                                                                                \
     hipLaunchKernelGGL((mlstm_scan_kernel<TT, DD>), grid, block, lds, st, o_raw, (const TT*)proj, p_stride, i_bias,  \
-                       f_bias, state_nm, state_s, qsl, seq_lens, slot_table, st_stride, H, D, Dv, Dn, LPC, cap);     \
+                       f_bias, state_nm, state_s, qsl, seq_lens, slot_table, st_stride, H, D, Dv, Dn, LPC, TCH, cap);     \
     hipLaunchKernelGGL((mlstm_out_kernel<TT>), dim3(T, H), dim3(64), 0, st, (TT*)out, o_stride, o_raw,               \
                        (const TT*)proj + gate_off, p_stride, weight, H, Dv, eps);                                    \
   } while (0)

@@ -59,9 +59,10 @@ _SIGS = {
     "vda_moe_topk_softmax": [P, P, P, I, I, I, I, L, I, P],
     "vda_moe_align": [P, P, P, I, I, P],
     "vda_residual_norms": [P, P, L, P, P, P, L, F, F, I, I, I, P],
-    "vda_latent_norm_rope_cache": [P, L, P, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "vda_latent_norm_rope_cache": [P, L, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "vda_latent_window_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, I, I, P],
     "vda_mlstm": [P, L, P, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P],
+    "vda_moe_pairs": [P, L, P, P, L, P, P, P, P, I, I, I, I, I, I, F, I, P],
     "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, F, P],
     "vda_moe_down": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
     "vda_moe_sum": [P, P, P, I, I, I, L, I, P],
@@ -82,7 +83,7 @@ _SIGS = {
     "vda_cb4_dequant_post": [P, P, P, P, I, I, I, I, I, P],
     "vda_w8_dequant": [P, P, P, P, I, I, I, I, P],
     "vda_mla_cache_write": [P, P, P, P, P, I, I, I, I, L, L, I, I, F, P],
-    "vda_mla_attention": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, L, L, F, I, I, F, P],
+    "vda_mla_attention": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, L, L, F, I, I, F, I, P],
     "vda_mla_supported": [I, I],
     "vda_lora_shrink": [P, P, P, P, I, I, I, L, I, P],
     "vda_lora_expand": [P, P, P, P, I, I, I, L, I, P],

@@ -549,7 +549,7 @@ def mla_cache_write(kv_c, k_pe, kc, vt, slot_mapping, kv_scale=1.0):
         vt[b, :, o] = kv_c[t].to(vt.dtype)
 
 
-def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale=1.0):
+def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale=1.0, window=0):
     T, H, DK = q.shape
     DV, BS = vt.shape[1], kc.shape[1]
     if kc.dtype != torch.float8_e4m3fn:
@@ -570,6 +570,8 @@ def mla_attention(q, kc, vt, block_table, seq_lens, q_start_loc, scale, kv_scale
         pos = torch.arange(L, device=q.device).view(1, 1, L)
         lim = (L - n + torch.arange(n, device=q.device) + 1).view(n, 1, 1)
         sc = sc.masked_fill(pos >= lim, float("-inf"))
+        if window > 0:
+            sc = sc.masked_fill(pos < lim - window, float("-inf"))
         out[a:b] = torch.einsum("nhl,ld->nhd", torch.softmax(sc, dim=-1), V).to(q.dtype)
     return out
 
@@ -705,7 +707,7 @@ def rotate_interleaved(x, cos, sin):
 
 
 def latent_norm_rope_cache(q, down, c_weight, cos_sin, positions, qf, kc, slot_mapping, H: int, D: int, P: int,
-                           R: int, rot_dims: int, eps: float):
+                           R: int, rot_dims: int, eps: float, vt=None):
     """q [T, H * (D + P)], down [T, R + P]; cos_sin fp32 [positions, rot_dims] (cosines then sines).
     Cache row of a token = [rms(down[:R]) * c_weight | rotated down[R:]] -> kc [blocks, bs, R + P] at slot_mapping;
     the rotated last P values of every query head go to qf[:, h, R:] (qf [T, H, R + P])."""
@@ -725,6 +727,8 @@ def latent_norm_rope_cache(q, down, c_weight, cos_sin, positions, qf, kc, slot_m
         ok = slot_mapping[:T] >= 0
         sl = slot_mapping[:T][ok].long()
         kc[sl // bs, sl % bs] = torch.cat([c, kr], -1)[ok].to(kc.dtype)
+        if vt is not None and vt.numel():
+            vt[sl // bs, :, sl % bs] = c[ok].to(vt.dtype)
 
 
 def latent_window_attention(q, kc, block_table, seq_lens, qsl, scale: float, window: int, R: int):

@@ -14,7 +14,7 @@ from typing import Any, Callable, NamedTuple, Optional
 
 from ..logger import init_logger
 from ..parallel.utils import cdiv
-from .kv_cache_interface import (FullAttentionSpec, KVCacheConfig, KVCacheGroupSpec, KVCacheSpec,
+from .kv_cache_interface import (FullAttentionSpec, KVCacheConfig, KVCacheGroupSpec, KVCacheSpec, MLASpec,
                                  KVCacheTensor, SlidingWindowSpec)
 
 logger = init_logger(__name__)
@@ -176,10 +176,10 @@ def get_kv_cache_config(vllm_config, spec: dict[str, KVCacheSpec], available: in
         nb = _num_blocks(vllm_config, available, page, len(names))
         tensors = [KVCacheTensor(size=page * nb, shared_by=[n]) for n in names]
         groups = [KVCacheGroupSpec(names, spec[names[0]])]
-    elif all(type(s_) is FullAttentionSpec and not s_.use_mla for s_ in spec.values()) \
+    elif all(type(s_) in (FullAttentionSpec, MLASpec) for s_ in spec.values()) \
             and len({s_.block_size for s_ in spec.values()}) == 1:
-        # full attention everywhere, but layers keep different numbers of KV heads (DeciLM / Nemotron-NAS): one
-        # group and one block table, every layer's tensor sized by its own page
+        # full attention everywhere, but layers keep different numbers of KV heads (DeciLM / Nemotron-NAS) or latent
+        # rows of different widths: one group and one block table, every layer's tensor sized by its own page
         total = sum(spec[n].page_size_bytes for n in names)
         nb = _num_blocks(vllm_config, available, total, 1)
         tensors = [KVCacheTensor(size=spec[n].page_size_bytes * nb, shared_by=[n]) for n in names]
