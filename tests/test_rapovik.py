@@ -137,7 +137,8 @@ def test_clamped_gated_pair(dev, dt, ff, limit):
 
 
 # sizes the MFMA kernel is built for (rows of 96 and 160 with 64 / 128 latent values) and sizes it is not
-LATENT_SIZES = [(3, 12, 8, 24, 9, 8), (4, 16, 32, 64, 40, 32), (2, 8, 32, 128, 17, 16), (5, 6, 6, 10, None, 4),
+LATENT_SIZES = [(3, 12, 8, 24, 9, 8), (4, 16, 32, 64, 40, 32), (2, 8, 32, 128, 17, 16), (8, 8, 32, 128, 30, 32),
+                (5, 6, 6, 10, None, 4),
                 (1, 4, 2, 6, 1, 0), (2, 8, 4, 12, 33, 4)]
 
 
@@ -299,26 +300,30 @@ def test_mamba2_mixer_pieces(dev, H, E, N, G, taps, parts):
         y = ops.selective_scan(xbc[:, :inner], p[:, inner + ch:].contiguous(), A, B, C, P["D"].to(dev),
                                p[:, :inner], P["dt_bias"].to(dev), state, qsl, sl, tbl, softplus=True, num_groups=G,
                                max_query_len=n)
-        f = y.float().view(n, parts, -1)
-        f = f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + eps)
-        got.append((f.view(n, -1) * P["norm"].to(dev)).cpu())
+        got.append(ops.group_rms_norm(y, P["norm"].to(dev), eps, parts).cpu())
         done += n
     assert rel(torch.cat(got), want) < 3e-5
 
 
-@pytest.mark.parametrize("E,top,count,keep", [(6, 2, 3, 2), (8, 3, 2, 1), (5, 1, 1, 1), (12, 4, 4, 2), (4, 2, 4, 3)])
-def test_group_limited_choice(E, top, count, keep):
+@pytest.mark.parametrize("dev", DEVICES)
+@pytest.mark.parametrize("E,top,count,keep", [(6, 2, 3, 2), (8, 3, 2, 1), (5, 1, 1, 1), (12, 4, 4, 2), (4, 2, 4, 3),
+                                              (192, 6, 8, 3), (70, 7, 1, 1)])
+def test_group_limited_choice(dev, E, top, count, keep):
     """Choice by score + bias inside the best groups only; weights are the plain scores.  Biases push choice scores
-    below zero, so a left-out group must count as minus infinity, not as zero."""
+    below zero, so a left-out group must count as minus infinity, not as zero.  On the GPU the one-launch kernel."""
     from vllm_distributed_amd.layers.moe import grouped_topk
     T, Wd = 64, 16
     h = torch.randn(T, Wd)
     w = {"router": torch.randn(E, Wd), "correction": torch.randn(E) - 1.5}
     ids, wts = O.route(h, w, {"experts": E, "top": top, "groups": {"count": count, "keep": keep}})
-    assert ((torch.sigmoid(h @ w["router"].T) + w["correction"]) < 0).any()
-    gw, gi = grouped_topk(torch.sigmoid(h @ w["router"].T), top, False, count, keep, w["correction"])
+    logits = h @ w["router"].T
+    assert ((torch.sigmoid(logits) + w["correction"]) < 0).any()
+    routed = ops.moe_grouped_sigmoid_topk(logits.to(dev), w["correction"].to(dev), top, count, keep, False)
+    assert (routed is not None) == (dev == "cuda")
+    gw, gi = routed if routed is not None else grouped_topk(torch.sigmoid(logits), top, False, count, keep,
+                                                            w["correction"])
     a = torch.zeros(T, E).scatter_(1, ids, wts)
-    b = torch.zeros(T, E).scatter_(1, gi.long(), gw)
+    b = torch.zeros(T, E).scatter_(1, gi.long().cpu(), gw.cpu())
     torch.testing.assert_close(a, b)
 
 

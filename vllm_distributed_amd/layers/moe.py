@@ -206,6 +206,12 @@ class FusedMoE(nn.Module):
         if self.custom_routing_function is not None:
             w, ids = self.custom_routing_function(router_logits, k, self.renormalize)
             return w.float(), ids.to(torch.int32)
+        if self.use_grouped_topk and self.scoring_func == "sigmoid" and self.e_score_correction_bias is not None:
+            # one launch: scores, group scores, the groups that stay, the choice and its weights
+            routed = ops.moe_grouped_sigmoid_topk(router_logits, self.e_score_correction_bias, k,
+                                                  self.num_expert_group, self.topk_group, self.renormalize)
+            if routed is not None:
+                return routed
         if self.use_grouped_topk:
             scores = torch.softmax(router_logits.float(), -1) if self.scoring_func == "softmax" \
                 else torch.sigmoid(router_logits.float())

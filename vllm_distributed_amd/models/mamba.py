@@ -243,10 +243,7 @@ class Mamba2Mixer(StateSpaceLayer):
         # y already carries the silu(gate) factor (applied inside the scan kernel)
         if not self.use_norm:
             return y
-        T = y.shape[0]
-        f = y.float().view(T, self.norm_groups, -1)
-        f = f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + self.norm_eps)
-        return (f.view(T, -1) * self.norm_weight.float()).to(y.dtype)
+        return ops.group_rms_norm(y, self.norm_weight, self.norm_eps, self.norm_groups)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         md = get_forward_context().attn_metadata

@@ -98,7 +98,7 @@ class RapovikMoE(nn.Module):
         count, keep = int(groups.get("count", 1) or 1), int(groups.get("keep", 1) or 1)
         if E % count or keep > count or top > (E // count) * keep:
             raise ValueError(f"{prefix}: {E} experts, {count} groups (keep {keep}) and top {top} do not fit")
-        self.router = ReplicatedLinear(width, E, bias=False, prefix=f"{prefix}.router")
+        self.router = ReplicatedLinear(width, E, bias=False, params_dtype=torch.float32, prefix=f"{prefix}.router")
         self.correction = _fp32_param((E,), 0.0)
         self.experts = FusedMoE(E, top, width, int(ex["ff"]), renormalize=False, use_grouped_topk=True,
                                 num_expert_group=count, topk_group=keep, quant_config=quant_config,
@@ -110,7 +110,7 @@ class RapovikMoE(nn.Module):
                                act_limit=float(sh["limit"])) if sh else None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        logits = F.linear(x.float(), self.router.weight.float())          # the router runs in fp32
+        logits = F.linear(x.float(), self.router.weight)                  # the router runs in fp32
         out = self.experts(x, logits)
         return out + self.shared(x) if self.shared is not None else out
 

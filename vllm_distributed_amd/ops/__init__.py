@@ -869,6 +869,37 @@ def moe_topk_softmax(logits: torch.Tensor, k: int, renormalize: bool = True):
     return w, ids
 
 
+def moe_grouped_sigmoid_topk(logits: torch.Tensor, bias: Optional[torch.Tensor], k: int, groups: int, keep: int,
+                             renormalize: bool):
+    """Group-limited choice with sigmoid scores: choice = sigmoid(logits) + bias; a group of neighbouring experts scores
+    the sum of its two largest choices; the k best choices inside the ``keep`` best groups win, weighted by their
+    plain sigmoid (renormalised on request).  Returns (weights f32 [T, k], ids i32 [T, k]); None when the kernel does
+    not take the sizes (the caller then runs the PyTorch form)."""
+    T, E = logits.shape
+    if not _dev(logits) or E > 512 or k > 64 or groups > 64 or E % groups or logits.stride(1) != 1 \
+            or logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        return None
+    w = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((T, k), dtype=torch.int32, device=logits.device)
+    assert bias is None or (bias.dtype == torch.float32 and bias.is_contiguous())
+    N.call("vda_moe_grouped_sigmoid_topk", w.data_ptr(), ids.data_ptr(), logits.data_ptr(), N.ptr(bias), T, E, k,
+           groups, keep, int(renormalize), logits.stride(0), N.dt(logits.dtype), N.stream())
+    return w, ids
+
+
+def group_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int) -> torch.Tensor:
+    """RMS norm over ``groups`` equal parts of every row, each part by its own root mean square, times weight."""
+    T, W = x.shape
+    if not _dev(x) or x.stride(1) != 1 or weight.dtype not in (x.dtype, torch.float32):
+        f = x.float().view(T, groups, -1)
+        f = f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + eps)
+        return (f.view(T, -1) * weight.float()).to(x.dtype)
+    out = torch.empty((T, W), dtype=x.dtype, device=x.device)
+    N.call("vda_group_rms_norm", out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), weight.data_ptr(),
+           float(eps), T, W, groups, N.dt(x.dtype), N.dt(weight.dtype), N.stream())
+    return out
+
+
 def moe_grouped_ok(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> bool:
     I = w13.shape[1] // 2
     return (x.dtype in (torch.bfloat16, torch.float16) and w13.shape[2] % 128 == 0 and I % 128 == 0

@@ -85,6 +85,9 @@ struct MlaParams {
   float scale;              // softmax scale, times the cache scale for an fp8 cache
   float v_scale;            // 1, or the cache scale for an fp8 cache
   int window;               // > 0: a query at position i sees the keys j with 0 <= i - j < window
+  int wave_cols;            // 1: every wave takes 16 columns of its own over all keys (prompts: neighbouring tokens
+                            //    walk the same keys at the same time, so the rows come from the cache near the CU);
+                            // 0: the 4 waves share 16 columns and split the keys (few query tokens)
 };
 
 template <typename T, int DK, int DV, bool F8>
@@ -103,8 +106,9 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
   const int qs = p.q_start_loc[seq];
   const int q_len = p.q_start_loc[seq + 1] - qs;
   const int seq_len = p.seq_lens[seq];
-  const int c0 = blockIdx.y * 16;                    // first (token, head) column of this workgroup
-  if (seq_len <= 0 || c0 >= q_len * p.H) return;
+  // first (token, head) column of this workgroup, or of this wave
+  const int c0 = p.wave_cols ? (blockIdx.y * 4 + wave) * 16 : blockIdx.y * 16;
+  if (seq_len <= 0 || c0 >= q_len * p.H) return;       // wave_cols: no barrier follows, waves may leave alone
   const int ctx = seq_len - q_len;
   const int BS = p.BS;
   const int* bt = p.block_table + (long)seq * p.max_blocks;
@@ -145,7 +149,7 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
   const int krow0 = 8 * (r >> 2) + (r & 3);     // tile u, row r <-> key 8*(r>>2) + 4u + (r&3) of the step
   const float sc = p.scale * 1.4426950408889634f;
 
-  for (int step = a0 + wave; step < step_hi; step += 4) {
+  for (int step = p.wave_cols ? a0 : a0 + wave; step < step_hi; step += p.wave_cols ? 1 : 4) {
     const int tb = step * 32 + 8 * g;            // first of this lane's 8 keys
     f32x4 s2[2];
 #pragma unroll
@@ -200,7 +204,7 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
   // ---- merge the 4 waves into wave 0, one sender at a time (one staging buffer keeps LDS at NT KB) ----
   __shared__ f32x4 s_acc[NT][64];
   __shared__ float s_ml[2][64];
-  for (int snd = 1; snd < 4; ++snd) {
+  for (int snd = 1; snd < 4 && !p.wave_cols; ++snd) {
     if (wave == snd) {
       s_ml[0][lane] = m;
       s_ml[1][lane] = l;
@@ -220,7 +224,7 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
     }
     __syncthreads();
   }
-  if (wave != 0 || !valid) return;
+  if ((wave != 0 && !p.wave_cols) || !valid) return;
   const float inv = l > 0.f ? p.v_scale / l : 0.f;
   const long tok = qs + ti;
   if (p.nsplit == 1) {
@@ -287,7 +291,7 @@ __global__ __launch_bounds__(64) void mla_reduce_kernel(T* out, const float* par
 
 template <typename T, int DK, int DV>
 static int launch_mla(const MlaParams& p, int S, int T_tokens, int max_q, bool f8, hipStream_t st) {
-  dim3 block(256), grid(S, (max_q * p.H + 15) / 16, p.nsplit);
+  dim3 block(256), grid(S, p.wave_cols ? (max_q * p.H + 63) / 64 : (max_q * p.H + 15) / 16, p.nsplit);
   if (f8) hipLaunchKernelGGL((mla_attention_kernel<T, DK, DV, true>), grid, block, 0, st, p);
   else hipLaunchKernelGGL((mla_attention_kernel<T, DK, DV, false>), grid, block, 0, st, p);
   if (p.nsplit > 1)
@@ -315,6 +319,7 @@ VDA_EXPORT int vda_mla_attention(void* out, const void* q, const void* kc, const
   p.q_stride = q_stride; p.out_stride = out_stride;
   p.scale = scale * (kv_fp8 ? kv_scale : 1.f); p.v_scale = kv_fp8 ? kv_scale : 1.f;
   p.window = window > 0 ? window : 0;
+  p.wave_cols = (nsplit == 1 && (long)max_q * H >= 64) ? 1 : 0;
   const bool f8 = kv_fp8 != 0;
 #define BYD(TT) do { if (DK == 576) launch_mla<TT, 576, 512>(p, S, T_tokens, max_q, f8, st);      \
                      else if (DK == 96) launch_mla<TT, 96, 64>(p, S, T_tokens, max_q, f8, st);    \

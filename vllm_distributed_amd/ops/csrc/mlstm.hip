@@ -156,7 +156,7 @@ VDA_EXPORT int vda_mlstm(void* out, long o_stride, float* o_raw, const void* pro
   if (T <= 0 || S <= 0) return 0;
   if (H <= 0 || D <= 0 || Dv <= 0 || Dn < D + 1) return -1;
   int LPC = 1;
-  while ((D + LPC - 1) / LPC > 32 && LPC < 64) LPC <<= 1;
+  while ((D + LPC - 1) / LPC > 16 && LPC < 64) LPC <<= 1;      // 16 state values per lane: short steps, many lanes
   const int per = (D + LPC - 1) / LPC;
   if (per > 32) return -2;                       // D beyond 2048
   const int DPT = per <= 8 ? 8 : per <= 16 ? 16 : 32;

@@ -72,6 +72,120 @@ __global__ __launch_bounds__(256) void moe_topk_softmax_kernel(float* __restrict
   }
 }
 
+// Group-limited choice with sigmoid scores and a selection bias (DeepSeek-V3 style routing), one wave per token:
+//   s = sigmoid(logit);  choice = s + bias;  experts form `groups` equal groups of neighbours, a group's score is the
+//   sum of its two largest choice scores (its largest when it has one member); only the `keep` best groups stay in the
+//   race (the others count as minus infinity); the k largest choice scores win and are weighted by their plain s
+//   (divided by the winners' sum when renorm is set).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_grouped_sigmoid_topk_kernel(
+    float* __restrict__ topk_w, int* __restrict__ topk_id, const T* __restrict__ logits,
+    const float* __restrict__ bias, int num_tokens, int E, int k, int groups, int keep, int renorm, long stride) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= num_tokens) return;
+  constexpr int PER = 8;                 // up to 512 experts
+  const int gs = E / groups;
+  float s[PER], c[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = lane + 64 * i;
+    const float z = e < E ? (float)logits[(long)t * stride + e] : 0.f;
+    s[i] = 1.f / (1.f + expf(-z));
+    c[i] = e < E ? s[i] + (bias ? bias[e] : 0.f) : -INFINITY;
+    if (!(c[i] == c[i])) c[i] = -INFINITY;          // NaN logits (warm-up runs over empty contexts)
+  }
+  if (groups > 1) {
+    // lane g ends up with the score of group g
+    float gscore = -INFINITY;
+    for (int g = 0; g < groups; ++g) {
+      float m1 = -INFINITY, m2 = -INFINITY;          // this lane's two largest members of group g
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int e = lane + 64 * i;
+        if (e < E && e / gs == g) {
+          if (c[i] > m1) { m2 = m1; m1 = c[i]; }
+          else if (c[i] > m2) m2 = c[i];
+        }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {            // merge two (largest, second) pairs
+        const float a1 = __shfl_xor(m1, o, 64), a2 = __shfl_xor(m2, o, 64);
+        const float hi = fmaxf(m1, a1);
+        m2 = fmaxf(fminf(m1, a1), fmaxf(m2, a2));
+        m1 = hi;
+      }
+      const float sc = gs > 1 ? m1 + m2 : m1;
+      if (lane == g) gscore = sc;
+    }
+    unsigned long long allowed = 0ull;
+    for (int j = 0; j < keep; ++j) {
+      float best = (lane < groups && !((allowed >> lane) & 1ull)) ? gscore : -INFINITY;
+      int bi = (lane < groups && !((allowed >> lane) & 1ull)) ? lane : 0x7fffffff;
+      if (!(best > -INFINITY)) bi = 0x7fffffff;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+      }
+      if (bi == 0x7fffffff) break;                   // wave-uniform
+      allowed |= 1ull << bi;
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && !((allowed >> (e / gs)) & 1ull)) c[i] = -INFINITY;
+    }
+  }
+  float picked = 0.f, my_w = 0.f;
+  int my_id = 0;
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY, bs = 0.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      if (c[i] > best) { best = c[i]; bs = s[i]; bi = lane + 64 * i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64), os = __shfl_xor(bs, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bs = os; bi = oi; }
+    }
+    if (bi == 0x7fffffff) { bi = j; bs = 0.f; }      // no candidate left: a valid, distinct id with weight 0
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (lane + 64 * i == bi) c[i] = -INFINITY;
+    picked += bs;
+    if (lane == j) { my_w = bs; my_id = bi; }
+  }
+  if (lane < k) {
+    const float scale = renorm ? (picked > 0.f ? 1.f / picked : 0.f) : 1.f;
+    topk_w[(long)t * k + lane] = my_w * scale;
+    topk_id[(long)t * k + lane] = my_id;
+  }
+}
+
+VDA_EXPORT int vda_moe_grouped_sigmoid_topk(float* topk_w, int* topk_id, const void* logits, const float* bias,
+                                            int num_tokens, int E, int k, int groups, int keep, int renorm,
+                                            long stride, int dtype, hipStream_t st) {
+  if (num_tokens <= 0) return 0;
+  if (E < 1 || E > 512 || k < 1 || k > 64 || k > E || groups < 1 || groups > 64 || E % groups || keep < 1 ||
+      keep > groups)
+    return -1;
+  dim3 grid((num_tokens + 3) / 4), block(256);
+#define L(TT) hipLaunchKernelGGL((moe_grouped_sigmoid_topk_kernel<TT>), grid, block, 0, st, topk_w, topk_id,          \
+                                 (const TT*)logits, bias, num_tokens, E, k, groups, keep, renorm, stride)
+  if (dtype == VDA_BF16) L(bf16_t);
+  else if (dtype == VDA_F16) L(f16_t);
+  else if (dtype == VDA_F32) L(float);
+  else return -3;
+#undef L
+  VDA_CHECK_LAUNCH();
+  return 0;
+}
+
 VDA_EXPORT int vda_moe_topk_softmax(float* topk_w, int* topk_id, const void* logits, int num_tokens, int E, int k,
                                     int renorm, long stride, int dtype, hipStream_t st) {
   if (E > 512 || k > 64 || k > E || num_tokens < 0) return -1;

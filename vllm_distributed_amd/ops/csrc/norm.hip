@@ -200,40 +200,97 @@ VDA_EXPORT int vda_layer_norm(void* out, const void* in, const void* w, const vo
 //   h  = x / rms(x) * (off + w_pre)       (h given: the input of the next sub-layer)
 // One pass over the fp32 residual row per token: the write of one sub-layer and the read of the next are one launch,
 // the role add + RMSNorm fusion plays for 16-bit residuals.  Gains are fp32; `off` is 1 for gains stored around zero.
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void residual_norms_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                              long y_stride, const float* __restrict__ w_post,
                                                              const float* __restrict__ w_pre, T* __restrict__ h,
                                                              long h_stride, float eps, float off, int W) {
+  // VEC consecutive values per thread and trip (4: rows whose width and strides are multiples of four)
   extern __shared__ float row[];          // the updated residual row
   __shared__ float red[16];
   const long t = blockIdx.x;
   const int tid = threadIdx.x;
   float* xr = x + t * W;
+  const T* yr = y ? y + t * y_stride : nullptr;
   float ry = 0.f;
   if (y) {
     float ss = 0.f;
-    for (int c = tid; c < W; c += 256) {
-      const float v = (float)y[t * y_stride + c];
-      ss += v * v;
+    for (int c = tid * VEC; c < W; c += 256 * VEC) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float v = (float)yr[c + i];
+        ss += v * v;
+      }
     }
     ss = block_sum(ss, red);
     ry = 1.f / sqrtf(ss / (float)W + eps);
   }
   float sx = 0.f;
-  for (int c = tid; c < W; c += 256) {
-    float v = xr[c];
-    if (y) {
-      v += (float)y[t * y_stride + c] * ry * (off + w_post[c]);
-      xr[c] = v;
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+    float v[VEC];
+    if (VEC == 4) {
+      const f32x4 q = *reinterpret_cast<const f32x4*>(xr + c);
+      v[0] = q[0]; v[1 % VEC] = q[1]; v[2 % VEC] = q[2]; v[3 % VEC] = q[3];
+    } else {
+      v[0] = xr[c];
     }
-    row[c] = v;
-    sx += v * v;
+    if (y) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[i] += (float)yr[c + i] * ry * (off + w_post[c + i]);
+      if (VEC == 4) *reinterpret_cast<f32x4*>(xr + c) = f32x4{v[0], v[1 % VEC], v[2 % VEC], v[3 % VEC]};
+      else xr[c] = v[0];
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      row[c + i] = v[i];
+      sx += v[i] * v[i];
+    }
   }
   if (!h) return;
   sx = block_sum(sx, red);
   const float rx = 1.f / sqrtf(sx / (float)W + eps);
-  for (int c = tid; c < W; c += 256) h[t * h_stride + c] = (T)(row[c] * rx * (off + w_pre[c]));
+  for (int c = tid * VEC; c < W; c += 256 * VEC) {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) h[t * h_stride + c + i] = (T)(row[c + i] * rx * (off + w_pre[c + i]));
+  }
+}
+
+// y[t, g, :] = x[t, g, :] / rms(x[t, g, :]) * weight[g, :] over `groups` equal parts of a row (fp32 inside)
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void group_rms_norm_kernel(T* __restrict__ out, long o_stride,
+                                                             const T* __restrict__ x, long x_stride,
+                                                             const TW* __restrict__ weight, float eps, int part) {
+  __shared__ float red[16];
+  const long t = blockIdx.x;
+  const int g = blockIdx.y, tid = threadIdx.x;
+  const T* xr = x + t * x_stride + (long)g * part;
+  float ss = 0.f;
+  for (int c = tid; c < part; c += 256) {
+    const float v = (float)xr[c];
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)part + eps);
+  for (int c = tid; c < part; c += 256)
+    out[t * o_stride + (long)g * part + c] = (T)((float)xr[c] * r * (float)weight[(long)g * part + c]);
+}
+
+VDA_EXPORT int vda_group_rms_norm(void* out, long o_stride, const void* x, long x_stride, const void* weight,
+                                  float eps, int T, int W, int groups, int dtype, int wdtype, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (groups < 1 || W % groups) return -1;
+  dim3 grid(T, groups), block(256);
+#define L(TT, TW) hipLaunchKernelGGL((group_rms_norm_kernel<TT, TW>), grid, block, 0, st, (TT*)out, o_stride,       \
+                                     (const TT*)x, x_stride, (const TW*)weight, eps, W / groups)
+  if (dtype == VDA_BF16 && wdtype == VDA_BF16) L(bf16_t, bf16_t);
+  else if (dtype == VDA_BF16 && wdtype == VDA_F32) L(bf16_t, float);
+  else if (dtype == VDA_F16 && wdtype == VDA_F16) L(f16_t, f16_t);
+  else if (dtype == VDA_F16 && wdtype == VDA_F32) L(f16_t, float);
+  else if (dtype == VDA_F32 && wdtype == VDA_F32) L(float, float);
+  else return -3;
+#undef L
+  VDA_CHECK_LAUNCH();
+  return 0;
 }
 
 VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const float* w_post, const float* w_pre,
@@ -243,13 +300,16 @@ VDA_EXPORT int vda_residual_norms(float* x, const void* y, long y_stride, const 
   if ((y && !w_post) || (h && !w_pre)) return -1;
   const size_t lds = (size_t)W * 4;
   if (lds > 60 * 1024) return -2;
-#define L(TT) hipLaunchKernelGGL((residual_norms_kernel<TT>), dim3(T), dim3(256), lds, st, x, (const TT*)y, y_stride, \
-                                 w_post, w_pre, (TT*)h, h_stride, eps, off, W)
+  const bool vec = W % 4 == 0 && y_stride % 4 == 0 && h_stride % 4 == 0;
+#define L2(TT, VV) hipLaunchKernelGGL((residual_norms_kernel<TT, VV>), dim3(T), dim3(256), lds, st, x, (const TT*)y, \
+                                      y_stride, w_post, w_pre, (TT*)h, h_stride, eps, off, W)
+#define L(TT) do { if (vec) L2(TT, 4); else L2(TT, 1); } while (0)
   if (dtype == VDA_BF16) L(bf16_t);
   else if (dtype == VDA_F16) L(f16_t);
   else if (dtype == VDA_F32) L(float);
   else return -3;
 #undef L
+#undef L2
   VDA_CHECK_LAUNCH();
   return 0;
 }

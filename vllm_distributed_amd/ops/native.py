@@ -62,6 +62,8 @@ _SIGS = {
     "vda_latent_norm_rope_cache": [P, L, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "vda_latent_window_attention": [P, P, P, P, L, P, P, F, I, I, I, I, I, I, I, I, P],
     "vda_mlstm": [P, L, P, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P],
+    "vda_moe_grouped_sigmoid_topk": [P, P, P, P, I, I, I, I, I, I, L, I, P],
+    "vda_group_rms_norm": [P, L, P, L, P, F, I, I, I, I, I, P],
     "vda_moe_pairs": [P, L, P, P, L, P, P, P, P, I, I, I, I, I, I, F, I, P],
     "vda_moe_gate_up": [P, P, P, P, P, P, I, I, I, I, I, L, I, I, I, I, F, P],
     "vda_moe_down": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
