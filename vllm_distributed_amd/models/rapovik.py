@@ -170,7 +170,7 @@ class RapovikForCausalLM(nn.Module):
     # recurrent states live in per-row slots even when no layer is an attention layer
     row_state_slots = True
     # kernels outside the common set that this model launches (ops/build.py builds them on first use)
-    native_sources = ("latent_attention.hip", "mlstm.hip", "mamba.hip", "moe.hip", "gemm_tile.hip")
+    native_sources = ("latent_attention.hip", "mla.hip", "mlstm.hip", "mamba.hip", "moe.hip", "gemm_tile.hip")
 
     def __init__(self, vllm_config: VllmConfig, prefix: str = ""):
         super().__init__()
