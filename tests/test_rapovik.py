@@ -328,7 +328,7 @@ def test_group_limited_choice(dev, E, top, count, keep):
 
 
 @pytest.mark.parametrize("dev,dt", OP_CASES)
-@pytest.mark.parametrize("Wd,ff,E,k", [(48, 20, 6, 2), (72, 9, 5, 1), (256, 128, 4, 2)])
+@pytest.mark.parametrize("Wd,ff,E,k", [(48, 20, 6, 2), (72, 9, 5, 1), (256, 128, 4, 2), (128, 192, 3, 2)])
 def test_routed_experts_of_any_width(dev, dt, Wd, ff, E, k):
     T, limit = 21, 1.5
     x = torch.randn(T, Wd).to(dt)
@@ -362,6 +362,10 @@ VARIANTS = {
                                O.mamba_layer(heads=6, vdim=4, state=32, groups=3, conv=5, norm_groups=3)], loop=(0, 1, 2)),
     "mlstm_only": dict(layers=[O.mlstm_layer(heads=1, dim=40, vdim=8, gate_cap=4.0, mlp=None),
                                O.mlstm_layer(heads=3, dim=5, vdim=70)], loop=(1, 2, 2)),
+    "odd_widths": dict(layers=[O.attention_layer(heads=2, dim=6, rot_dim=32, vdim=6, kv_rank=64, window=5, rot_dims=4),
+                               O.mamba_layer(heads=3, vdim=6, state=10, groups=3, conv=3, norm_groups=1),
+                               O.attention_layer(heads=3, dim=5, rot_dim=6, vdim=7, kv_rank=9, window=4, mlp="moe"),
+                               O.mlstm_layer(heads=2, dim=7, vdim=9, mlp=None)], width=44, vocab=37, loop=(0, 2, 2)),
     "experts_plain": dict(layers=[O.mlstm_layer(mlp=O.feed_forward("moe", experts=5, top=1, groups=None, shared=None)),
                                   O.attention_layer(mlp=O.feed_forward("moe", experts=4, top=2, groups=(4, 3),
                                                                        shared=8))], width=40, vocab=50),

@@ -248,6 +248,166 @@ __global__ __launch_bounds__(256) void mla_attention_kernel(MlaParams p) {
   }
 }
 
+// ---- prompts: key / value tiles staged in LDS for four column groups ---------------------------------------------
+// One workgroup = 64 consecutive (token, head) columns of one sequence, 16 per wave.  Every 32-key step is copied
+// from the cache into LDS once (the latent rows in the order the MFMA row tiles want them, the transposed latent as
+// it lies) and read from there by all four waves: a quarter of the cache traffic of the form above, and the A
+// operands come from LDS instead of waiting on the cache one MFMA at a time.  Everything else -- operand layouts,
+// online softmax, masks -- is the form above; a wave skips the steps outside its own columns' range.
+template <typename T, int DK, int DV>
+__global__ __launch_bounds__(256) void mla_prefill_kernel(MlaParams p) {
+  using V8 = typename Vec<T>::v8;
+  using V4 = typename Vec<T>::v4;
+  constexpr int KS = DK / 32, NT = DV / 16, DQ = DK / 4;
+  constexpr int KROW = DK + 8;       // padded LDS rows: consecutive rows fall into different 16-byte bank groups
+  constexpr int VROW = 32 + 8;
+  static_assert(DK % 32 == 0 && DV % 16 == 0 && DQ % 8 == 0, "unsupported latent sizes");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* ks = reinterpret_cast<T*>(smem);                 // [32][KROW]: row u * 16 + r holds key 8 (r >> 2) + 4 u + (r & 3)
+  T* vs = ks + 32 * KROW;                             // [DV][VROW]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int seq = blockIdx.x;
+  const int qs = p.q_start_loc[seq];
+  const int q_len = p.q_start_loc[seq + 1] - qs;
+  const int seq_len = p.seq_lens[seq];
+  const int cw = blockIdx.y * 64;                    // first column of the workgroup
+  if (seq_len <= 0 || cw >= q_len * p.H) return;     // the whole workgroup leaves
+  const int ctx = seq_len - q_len;
+  const int BS = p.BS;
+  const int* bt = p.block_table + (long)seq * p.max_blocks;
+  const int nblk_valid = (seq_len + BS - 1) / BS;
+
+  // this lane's query column
+  const int c = cw + wave * 16 + r;
+  const int ti = c / p.H, head = c % p.H;
+  const bool valid = ti < q_len;
+  const int limit = valid ? ctx + ti + 1 : 0;
+  const int first = p.window > 0 ? max(limit - p.window, 0) : 0;
+  V8 qf[KS];
+  {
+    const T* qp = (const T*)p.q + (long)(qs + (valid ? ti : 0)) * p.q_stride + (long)head * DK + g * DQ;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = valid ? ld16<V8>(qp + 8 * s) : V8{};
+  }
+  int hi = limit, lo = valid ? first : 0x7fffffff;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    hi = max(hi, __shfl_xor(hi, o, 64));
+    lo = min(lo, __shfl_xor(lo, o, 64));
+  }
+  const int my_hi = (hi + 31) / 32, my_lo = min(lo / 32, my_hi);      // this wave's steps
+  // the workgroup's steps, from its first and last token (the same in every wave)
+  const int t_first = cw / p.H, t_last = min((cw + 63) / p.H, q_len - 1);
+  const int wg_hi = (ctx + t_last + 1 + 31) / 32;
+  const int wg_lo = p.window > 0 ? max(ctx + t_first + 1 - p.window, 0) / 32 : 0;
+
+  float m = -INFINITY, l = 0.f;
+  f32x4 acc[NT];
+#pragma unroll
+  for (int n = 0; n < NT; ++n) acc[n] = f32x4{0, 0, 0, 0};
+  const T* kc = (const T*)p.kc;
+  const T* vt = (const T*)p.vt;
+  const float sc = p.scale * 1.4426950408889634f;
+
+  for (int step = wg_lo; step < wg_hi; ++step) {
+    __syncthreads();                                   // the tiles of the step before are read
+    // the pages this step touches, looked up once (the same for every lane); a thread copies pieces of ONE latent
+    // row (8 threads per row) and of ONE 8-key column of the transposed tile, so that pages and row addresses are
+    // worked out once per step; all loads of a tile are in flight together before the first store to LDS
+    const int b0 = step * 32 / BS;
+    int pg[5];
+#pragma unroll
+    for (int j = 0; j < 5; ++j) pg[j] = bt[max(min(b0 + j, nblk_valid - 1), 0)];
+    auto page = [&](int tok) {
+      const int j = tok / BS - b0;
+      return j == 0 ? pg[0] : j == 1 ? pg[1] : j == 2 ? pg[2] : j == 3 ? pg[3] : pg[4];
+    };
+    {
+      constexpr int CH = DK / 8, KI = (CH + 7) / 8;      // 16-byte pieces per row; pieces per thread
+      const int L = tid >> 3, c0 = tid & 7;
+      const int rr = L & 15, u = L >> 4;
+      const int tok = step * 32 + 8 * (rr >> 2) + 4 * u + (rr & 3);
+      const T* src = kc + ((long)page(tok) * BS + (tok % BS)) * DK + c0 * 8;
+      T* dst = ks + L * KROW + c0 * 8;
+      V8 tmp[KI];
+#pragma unroll
+      for (int i = 0; i < KI; ++i)
+        if (c0 + 8 * i < CH) tmp[i] = ld16<V8>(src + 64 * i);
+#pragma unroll
+      for (int i = 0; i < KI; ++i)
+        if (c0 + 8 * i < CH) st16<V8>(dst + 64 * i, tmp[i]);
+    }
+    {
+      constexpr int VI = (DV + 63) / 64;                 // rows per thread
+      const int ch = tid & 3, d0 = tid >> 2;
+      const int tok = step * 32 + 8 * ch;
+      const T* src = vt + ((long)page(tok) * DV + d0) * BS + (tok % BS);
+      T* dst = vs + d0 * VROW + ch * 8;
+      V8 tmp[VI];
+#pragma unroll
+      for (int i = 0; i < VI; ++i)
+        if (d0 + 64 * i < DV) tmp[i] = ld16<V8>(src + (long)64 * i * BS);
+#pragma unroll
+      for (int i = 0; i < VI; ++i)
+        if (d0 + 64 * i < DV) st16<V8>(dst + 64 * i * VROW, tmp[i]);
+    }
+    __syncthreads();
+    if (step < my_lo || step >= my_hi) continue;       // wave-uniform
+    const int tb = step * 32 + 8 * g;                  // first of this lane's 8 keys
+    f32x4 s2[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const T* kp = ks + (u * 16 + r) * KROW + g * DQ;
+      f32x4 s = {0, 0, 0, 0};
+#pragma unroll
+      for (int k = 0; k < KS; ++k) s = mfma16(ld16<V8>(kp + 8 * k), qf[k], s);
+      s2[u] = s;
+    }
+    float sv[8] = {s2[0][0], s2[0][1], s2[0][2], s2[0][3], s2[1][0], s2[1][1], s2[1][2], s2[1][3]};
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      sv[j] = (tb + j < limit && tb + j >= first) ? sv[j] * sc : -INFINITY;
+      mx = fmaxf(mx, sv[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = (m == -INFINITY) ? 1.f : fexp2(m - m_use);     // nothing summed yet: nothing to rescale
+    m = m_new;
+    float ps = 0.f;
+    V8 pb;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float e = fexp2(sv[j] - m_use);
+      ps += e;
+      pb[j] = (T)e;
+    }
+    l = l * alpha + ps;
+    const T* vp = vs + r * VROW + 8 * g;
+    if (__any(alpha != 1.f)) {                          // the running maximum moved in some column: rescale (rare
+#pragma unroll                                          //  after a column's first steps)
+      for (int n = 0; n < NT; ++n) acc[n] *= alpha;
+    }
+#pragma unroll
+    for (int n = 0; n < NT; ++n) acc[n] = mfma16(ld16<V8>(vp + n * 16 * VROW), pb, acc[n]);
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!valid) return;
+  const float inv = l > 0.f ? p.v_scale / l : 0.f;
+  T* op = (T*)p.out + (long)(qs + ti) * p.out_stride + (long)head * DV + 4 * g;
+#pragma unroll
+  for (int n = 0; n < NT; ++n) {
+    V4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (T)(acc[n][i] * inv);
+    *reinterpret_cast<V4*>(op + 16 * n) = o;
+  }
+}
+
 // merge split partials: one wave per (token, head)
 template <typename T, int DV>
 __global__ __launch_bounds__(64) void mla_reduce_kernel(T* out, const float* part_out, const float* part_lse, int H,
@@ -292,6 +452,19 @@ __global__ __launch_bounds__(64) void mla_reduce_kernel(T* out, const float* par
 template <typename T, int DK, int DV>
 static int launch_mla(const MlaParams& p, int S, int T_tokens, int max_q, bool f8, hipStream_t st) {
   dim3 block(256), grid(S, p.wave_cols ? (max_q * p.H + 63) / 64 : (max_q * p.H + 15) / 16, p.nsplit);
+  if (p.wave_cols && !f8) {
+    // prompts on a 16-bit cache: the LDS-staged form
+    constexpr int lds = (32 * (DK + 8) + DV * 40) * (int)sizeof(T);
+    static bool ready = false;          // one attribute call per instantiation
+    if (!ready && lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)mla_prefill_kernel<T, DK, DV>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return (int)e;
+      ready = true;
+    }
+    hipLaunchKernelGGL((mla_prefill_kernel<T, DK, DV>), grid, block, lds, st, p);
+    return 0;
+  }
   if (f8) hipLaunchKernelGGL((mla_attention_kernel<T, DK, DV, true>), grid, block, 0, st, p);
   else hipLaunchKernelGGL((mla_attention_kernel<T, DK, DV, false>), grid, block, 0, st, p);
   if (p.nsplit > 1)
@@ -321,13 +494,15 @@ VDA_EXPORT int vda_mla_attention(void* out, const void* q, const void* kc, const
   p.window = window > 0 ? window : 0;
   p.wave_cols = (nsplit == 1 && (long)max_q * H >= 64) ? 1 : 0;
   const bool f8 = kv_fp8 != 0;
-#define BYD(TT) do { if (DK == 576) launch_mla<TT, 576, 512>(p, S, T_tokens, max_q, f8, st);      \
-                     else if (DK == 96) launch_mla<TT, 96, 64>(p, S, T_tokens, max_q, f8, st);    \
-                     else launch_mla<TT, 160, 128>(p, S, T_tokens, max_q, f8, st); } while (0)
+  int rc = 0;
+#define BYD(TT) do { if (DK == 576) rc = launch_mla<TT, 576, 512>(p, S, T_tokens, max_q, f8, st);      \
+                     else if (DK == 96) rc = launch_mla<TT, 96, 64>(p, S, T_tokens, max_q, f8, st);    \
+                     else rc = launch_mla<TT, 160, 128>(p, S, T_tokens, max_q, f8, st); } while (0)
   if (dtype == VDA_BF16) BYD(bf16_t);
   else if (dtype == VDA_F16) BYD(f16_t);
   else return -3;
 #undef BYD
+  if (rc) return rc;
   VDA_CHECK_LAUNCH();
   return 0;
 }
