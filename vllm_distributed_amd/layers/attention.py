@@ -520,13 +520,21 @@ class MLAAttention(nn.Module):
             out = torch.empty((T, self.num_heads, self.dv), dtype=q.dtype, device=q.device)
             if n < T:
                 out[n:].zero_()
-            nsplit = 1
-            if md.max_query_len <= 4:           # few query tokens: split the keys so that the launch fills the chip
+            # the batch's leading decode sequences (few query tokens: the keys split over waves and workgroups), then
+            # its prompts and portions (key steps staged in LDS for several tokens), as the other attention layers do
+            nd, ndt, n_pre = md.num_decode_seqs, md.num_decode_tokens, md.num_prefill_seqs
+            kw = dict(kv_scale=self._kv_scale_float, window=self.sliding_window)
+            if nd > 0:
                 keys = min(self.max_model_len, self.sliding_window + 32) if self.sliding_window else self.max_model_len
-                nsplit = ops.decode_num_splits(S * max(self.num_heads // 16, 1), 1, keys)
-            ops.mla_attention(out[:n], q[:n], self.k_cache, self.v_cache, md.block_table[:S], md.seq_lens[:S],
-                              md.query_start_loc[:S + 1], self.scale, md.max_query_len, nsplit, self._kv_scale_float,
-                              window=self.sliding_window)
+                nsplit = ops.decode_num_splits(nd * max(self.num_heads // 16, 1), 1, keys)
+                ops.mla_attention(out[:ndt], q[:ndt], self.k_cache, self.v_cache, md.block_table[:nd],
+                                  md.seq_lens[:nd], md.query_start_loc[:nd + 1], self.scale,
+                                  md.max_decode_query_len, nsplit, **kw)
+            if n_pre > 0:
+                e = ndt + md.num_prefill_tokens
+                ops.mla_attention(out[ndt:e], q[ndt:e], self.k_cache, self.v_cache, md.block_table[nd:nd + n_pre],
+                                  md.seq_lens[nd:nd + n_pre], md.prefill_query_start_loc, self.scale,
+                                  md.max_query_len, 1, **kw)
             return out
         out = ops.latent_window_attention(q[:n], self.k_cache, md.block_table[:S], md.seq_lens[:S],
                                           md.query_start_loc[:S + 1], self.scale, self.sliding_window, self.dv,
