@@ -130,7 +130,7 @@ class RapovikLayer(nn.Module):
         elif kind == "mamba2":
             cfg = SimpleNamespace(hidden_size=width, num_heads=int(m["heads"]), head_dim=int(m["vdim"]),
                                   intermediate_size=int(m["heads"]) * int(m["vdim"]), state_size=int(m["state"]),
-                                  conv_kernel=int(m["conv"]), n_groups=int(m["groups"]), use_bias=False,
+                                  conv_kernel=int(m["conv"]), n_groups=int(m.get("groups", 1)), use_bias=False,
                                   use_conv_bias=True, gated_norm=True, layer_norm_epsilon=eps,
                                   gated_norm_groups=int(m.get("norm_groups", 1)), time_step_limit=None)
             self.mixer = Mamba2Mixer(cfg, f"{prefix}.mixer")
