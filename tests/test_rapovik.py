@@ -35,6 +35,22 @@ def hybrid_layers():
             O.mlstm_layer(heads=3, dim=20, vdim=8, gate_cap=6.0, mlp="moe")]
 
 
+def wide_latent_layers():
+    """Latent rows of the widths the MFMA attention kernel is built for (96 and 160 values), no routed experts."""
+    return [O.attention_layer(heads=4, dim=16, rot_dim=32, vdim=10, kv_rank=64, window=40, rot_dims=12),
+            O.mamba_layer(mlp="dense"),
+            O.attention_layer(heads=2, dim=8, rot_dim=32, vdim=12, kv_rank=128, window=9)]
+
+
+def recurrent_layers():
+    """No attention layer at all: the page pool is book-keeping only, every mixer lives in state slots."""
+    return [O.mamba_layer(heads=2, vdim=8, state=24, groups=1, conv=2, norm_groups=1, mlp="dense"),
+            O.mlstm_layer(heads=3, dim=5, vdim=70, mlp=None), O.mamba_layer()]
+
+
+LAYER_SETS = {"hybrid": hybrid_layers, "wide_latent": wide_latent_layers, "recurrent_only": recurrent_layers}
+
+
 # ---- driving the engine ------------------------------------------------------------------------------------------
 def run_schedule(folder, dtype, device, prompts, schedule, max_tokens, block_size=16, eager=True):
     """``schedule``: steps of (request, token count); every request ends when its tokens are used up.  Returns
@@ -414,10 +430,11 @@ def test_portions_down_to_two_tokens(tmp_path, dev, dtype, block_size):
 
 
 @pytest.mark.parametrize("dev,dtype", CASES)
-def test_unequal_requests_share_steps_and_reuse_pages_and_slots(tmp_path, dev, dtype):
+@pytest.mark.parametrize("layers", list(LAYER_SETS))
+def test_unequal_requests_share_steps_and_reuse_pages_and_slots(tmp_path, dev, dtype, layers):
     """Seven requests over four slots and a pool of 10 pages: portions beside single tokens, requests that sit out
     steps, pages and slots of finished requests taken by later ones."""
-    folder, cfg, W = model(tmp_path, hybrid_layers(), seed=8, loop=(1, 4, 2))
+    folder, cfg, W = model(tmp_path, LAYER_SETS[layers](), seed=8, loop=(1, 4, 2) if layers == "hybrid" else (0, 2, 2))
     V = cfg["vocab"]
     prompts = {"a": tokens(40, V, 1), "b": tokens(17, V, 2), "c": tokens(1, V, 3), "d": tokens(33, V, 4),
                "e": tokens(48, V, 5), "f": tokens(9, V, 6), "g": tokens(30, V, 7)}
@@ -517,10 +534,11 @@ def test_long_decoding_keeps_the_state(tmp_path):
 
 
 @pytest.mark.gpu
-def test_decode_graphs_equal_eager(tmp_path):
+@pytest.mark.parametrize("layers", list(LAYER_SETS))
+def test_decode_graphs_equal_eager(tmp_path, layers):
     """Single decoded tokens through captured graphs (several replays with other work between them) give the
     eager logits."""
-    folder, cfg, W = model(tmp_path, hybrid_layers(), seed=10, loop=(1, 4, 2))
+    folder, cfg, W = model(tmp_path, LAYER_SETS[layers](), seed=10, loop=(1, 4, 2) if layers == "hybrid" else None)
     V = cfg["vocab"]
     prompts = {"a": tokens(30, V, 1), "b": tokens(22, V, 2)}
     sched = [[("a", 10), ("b", 4)]] + [[("a", 1), ("b", 1)]] * 18 + [[("a", 2)]]
