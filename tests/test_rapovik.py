@@ -376,6 +376,7 @@ VARIANTS = {
                                            O.attention_layer(heads=2, dim=8, rot_dim=32, vdim=12, kv_rank=128)]),
     "mamba_only": dict(layers=[O.mamba_layer(heads=2, vdim=8, state=24, groups=1, conv=2, norm_groups=1, mlp=None),
                                O.mamba_layer(heads=6, vdim=4, state=32, groups=3, conv=5, norm_groups=3)], loop=(0, 1, 2)),
+    "one_tap": dict(layers=[O.mamba_layer(conv=1, mlp=None), O.mamba_layer(heads=2, vdim=4, state=16, groups=2, conv=8)]),
     "mlstm_only": dict(layers=[O.mlstm_layer(heads=1, dim=40, vdim=8, gate_cap=4.0, mlp=None),
                                O.mlstm_layer(heads=3, dim=5, vdim=70)], loop=(1, 2, 2)),
     "odd_widths": dict(layers=[O.attention_layer(heads=2, dim=6, rot_dim=32, vdim=6, kv_rank=64, window=5, rot_dims=4),

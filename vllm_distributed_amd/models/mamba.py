@@ -253,8 +253,14 @@ class Mamba2Mixer(StateSpaceLayer):
         if md is None or self.conv_state is None:
             return self.out_proj(self._gated_norm((xbc[:, :di] * gate).contiguous()))
         tbl = self.slot_table(md)
-        xbc = ops.causal_conv1d(xbc, self.conv_weight, self.conv_bias, self.conv_state, md.query_start_loc,
-                                md.seq_lens, tbl, md.max_query_len)
+        if self.d_conv == 1:          # one tap: no earlier inputs, nothing carried
+            f = xbc.float() * self.conv_weight.float().view(1, -1)
+            if self.conv_bias is not None:
+                f = f + self.conv_bias.float()
+            xbc = torch.nn.functional.silu(f).to(x.dtype)
+        else:
+            xbc = ops.causal_conv1d(xbc, self.conv_weight, self.conv_bias, self.conv_state, md.query_start_loc,
+                                    md.seq_lens, tbl, md.max_query_len)
         gn = self.n_groups * self.d_state
         xs, B, C = xbc[:, :di], xbc[:, di:di + gn], xbc[:, di + gn:]
         if self.d_state_padded != self.d_state:
